@@ -1,0 +1,337 @@
+// C ABI of libgnnhwc_hip.so (declared in include/gnnhwc.h): argument validation, launch planning,
+// element-type dispatch and the optional per-kernel event timing.
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <vector>
+
+#include "../../include/gnnhwc.h"
+#include "gn_host.h"
+
+namespace gn {
+namespace {
+
+thread_local char g_error[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int env_int(const char *name, int fallback) {
+  const char *v = getenv(name);
+  return (v && *v) ? atoi(v) : fallback;
+}
+
+int elem_size(int dtype) {
+  switch (dtype) {
+    case GN_F32: return 4;
+    case GN_F64: return 8;
+    case GN_F16: return 2;
+    case GN_BF16: return 2;
+    default: return 0;
+  }
+}
+const char *dtype_name(int dtype) {
+  static const char *names[] = {"f32", "f64", "f16", "bf16"};
+  return (dtype >= 0 && dtype < 4) ? names[dtype] : "?";
+}
+
+// Cut (N, R, C) into workgroup tiles.  `vec` is 16 / sizeof(T) for the 128-bit path or 1 for the
+// scalar path; `streams` is the number of activation-sized tensors a tile reads (1 forward, 2 backward).
+//
+// Chunk width: a workgroup reads `lpr` lane vectors (lpr * 16 bytes) of each row.  Narrow chunks mean
+// tall tiles for the same number of workgroups, and the per-tile partial results (one entry per group
+// or channel and tile) shrink with the number of row tiles; so the narrowest chunk that still covers
+// whole 128-byte lines, divides the row evenly and leaves no lane idle is preferred.
+// Rows per tile: chosen so that a large tensor yields about `target` workgroups and a small one still
+// yields as many workgroups as it has lane rows, down to one row per lane.
+Plan make_plan(int64_t N, int64_t R, int64_t C, int64_t G, int vec, int streams) {
+  static const int forced_lpr = env_int("GNNHWC_LPR", 0);
+  static const int forced_fwd_steps = env_int("GNNHWC_FWD_STEPS", 0);
+  static const int forced_bwd_steps = env_int("GNNHWC_BWD_STEPS", 0);
+  const int forced_steps = streams == 1 ? forced_fwd_steps : forced_bwd_steps;
+  static const int forced_target = env_int("GNNHWC_TARGET_BLOCKS", 0);
+  Plan p;
+  p.N = N; p.R = R; p.C = C;
+  p.G = (int)G;
+  p.D = (int)(C / G);
+  p.vec = vec;
+  p.cv = (int)(C / vec);
+  int lpr = 0;
+  if (forced_lpr > 0 && forced_lpr <= kBlock && forced_lpr <= p.cv) {
+    lpr = forced_lpr;
+  } else if (vec > 1) {
+    static const int preferred[] = {16, 32, 8, 64, 128, 256};
+    for (int d : preferred)
+      if (p.cv % d == 0) { lpr = d; break; }
+  }
+  if (lpr == 0) {  // no even cut into whole cache lines: take the whole row, or equal-ish chunks of a long one
+    const int nchunk = (p.cv + kBlock - 1) / kBlock;
+    lpr = (p.cv + nchunk - 1) / nchunk;
+  }
+  p.lpr = lpr;
+  p.nchunk = (p.cv + lpr - 1) / lpr;
+  p.rpi = kBlock / lpr;
+  const int64_t lane_rows = (R + p.rpi - 1) / p.rpi;  // steps needed to walk one sample
+  const int64_t units = N * p.nchunk * lane_rows;     // workgroups if each took a single step
+  const int64_t target = forced_target > 0 ? forced_target : kTargetBlocks;
+  int64_t k;
+  if (forced_steps > 0) {
+    k = forced_steps;
+  } else {
+    k = (units + target - 1) / target;
+    if (k < kUnroll) {
+      k = units / 512;
+      if (k < 1) k = 1;
+      if (k > kUnroll) k = kUnroll;
+    } else {
+      k = (k + kUnroll - 1) / kUnroll * kUnroll;
+    }
+  }
+  if (k > lane_rows) k = lane_rows;
+  p.tile_rows = (int)(k * p.rpi);
+  p.tiles = (int)((R + p.tile_rows - 1) / p.tile_rows);
+  p.nblocks = N * p.tiles * p.nchunk;
+  static const int debug = env_int("GNNHWC_DEBUG_PLAN", 0);
+  if (debug)
+    fprintf(stderr, "[gnnhwc] plan(%s) N=%lld R=%lld C=%lld G=%d D=%d vec=%d cv=%d lpr=%d nchunk=%d rpi=%d tile_rows=%d tiles=%d nblocks=%lld\n",
+            streams == 1 ? "fwd" : "bwd", (long long)N, (long long)R, (long long)C, p.G, p.D, p.vec, p.cv, p.lpr,
+            p.nchunk, p.rpi, p.tile_rows, p.tiles, (long long)p.nblocks);
+  return p;
+}
+
+int check_shape(int64_t N, int64_t R, int64_t C, int64_t G, int dtype) {
+  if (elem_size(dtype) == 0) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "unknown dtype code %d", dtype);
+  if (N < 0 || R < 0 || C <= 0 || G <= 0)
+    return fail(GNNHWC_ERR_INVALID_ARGUMENT, "invalid shape N=%lld R=%lld C=%lld G=%lld", (long long)N, (long long)R,
+                (long long)C, (long long)G);
+  if (C % G != 0)
+    return fail(GNNHWC_ERR_INVALID_ARGUMENT, "num_channels (%lld) must be divisible by num_groups (%lld)", (long long)C,
+                (long long)G);
+  if (C > (1 << 24) || N > ((int64_t)1 << 31) || R > ((int64_t)1 << 40) ||
+      (double)N * (double)R * (double)C > 4.0e18)
+    return fail(GNNHWC_ERR_INVALID_ARGUMENT, "shape N=%lld R=%lld C=%lld is beyond the supported index range",
+                (long long)N, (long long)R, (long long)C);
+  return GNNHWC_OK;
+}
+int check_dtypes(int dtype, int pdtype, int sdtype) {
+  const bool half = dtype == GN_F16 || dtype == GN_BF16;
+  if (!(pdtype == dtype || (half && pdtype == GN_F32)))
+    return fail(GNNHWC_ERR_INVALID_ARGUMENT,
+                "weight/bias dtype %s does not match data dtype %s (only f32 parameters with f16/bf16 data may differ)",
+                dtype_name(pdtype), dtype_name(dtype));
+  if (!(sdtype == dtype || (half && sdtype == GN_F32)))
+    return fail(GNNHWC_ERR_INVALID_ARGUMENT,
+                "mean/rstd dtype %s does not match data dtype %s (only f32 statistics with f16/bf16 data may differ)",
+                dtype_name(sdtype), dtype_name(dtype));
+  return GNNHWC_OK;
+}
+bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+size_t acc_size(int dtype) { return dtype == GN_F64 ? 8 : 4; }
+size_t fwd_ws_bytes(int64_t N, int64_t R, int64_t C, int64_t G, int dtype) {
+  const int vec = 16 / elem_size(dtype);
+  size_t need = fwd_workspace(make_plan(N, R, C, G, 1, 1)).total;
+  if (C % vec == 0) {
+    const size_t v = fwd_workspace(make_plan(N, R, C, G, vec, 1)).total;
+    if (v > need) need = v;
+  }
+  return need * acc_size(dtype);
+}
+size_t bwd_ws_bytes(int64_t N, int64_t R, int64_t C, int64_t G, int dtype) {
+  const int vec = 16 / elem_size(dtype);
+  size_t need = bwd_workspace(make_plan(N, R, C, G, 1, 2)).total;
+  if (C % vec == 0) {
+    const size_t v = bwd_workspace(make_plan(N, R, C, G, vec, 2)).total;
+    if (v > need) need = v;
+  }
+  return need * acc_size(dtype);
+}
+
+__global__ void fill_zero_kernel(void *p, int64_t n, int dtype) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  switch (dtype) {
+    case GN_F32: ((float *)p)[i] = 0.f; break;
+    case GN_F64: ((double *)p)[i] = 0.0; break;
+    default: ((uint16_t *)p)[i] = 0; break;
+  }
+}
+
+// ---- per-kernel event timing ----
+struct Timed {
+  int kind;
+  hipEvent_t start, stop;
+};
+thread_local bool g_profile = false;
+thread_local std::vector<Timed> g_timed;
+thread_local std::vector<hipEvent_t> g_event_pool;
+
+hipEvent_t get_event() {
+  if (!g_event_pool.empty()) {
+    hipEvent_t e = g_event_pool.back();
+    g_event_pool.pop_back();
+    return e;
+  }
+  hipEvent_t e = nullptr;
+  if (hipEventCreate(&e) != hipSuccess) return nullptr;
+  return e;
+}
+
+}  // namespace
+
+void profile_before(int kind, hipStream_t stream) {
+  if (!g_profile) return;
+  Timed t;
+  t.kind = kind;
+  t.start = get_event();
+  t.stop = get_event();
+  if (!t.start || !t.stop) return;
+  (void)hipEventRecord(t.start, stream);
+  g_timed.push_back(t);
+}
+void profile_after(int kind, hipStream_t stream) {
+  if (!g_profile || g_timed.empty() || g_timed.back().kind != kind) return;
+  (void)hipEventRecord(g_timed.back().stop, stream);
+}
+
+}  // namespace gn
+
+using namespace gn;
+
+extern "C" {
+
+int gnnhwc_version(void) { return (1 << 16) | 0; }
+
+const char *gnnhwc_last_error(void) { return g_error; }
+
+size_t gnnhwc_fwd_workspace_bytes(int64_t N, int64_t R, int64_t C, int64_t G, int dtype) {
+  if (check_shape(N, R, C, G, dtype) != GNNHWC_OK) return 0;
+  if (N == 0 || R == 0) return 256;
+  return align_up(fwd_ws_bytes(N, R, C, G, dtype), 256);
+}
+size_t gnnhwc_bwd_workspace_bytes(int64_t N, int64_t R, int64_t C, int64_t G, int dtype) {
+  if (check_shape(N, R, C, G, dtype) != GNNHWC_OK) return 0;
+  if (N == 0 || R == 0) return 256;
+  return align_up(bwd_ws_bytes(N, R, C, G, dtype), 256);
+}
+
+int gnnhwc_fwd(const void *x, const void *weight, const void *bias, void *y, void *mean, void *rstd, int64_t N,
+               int64_t R, int64_t C, int64_t G, double eps, int act, int dtype, int param_dtype, int stats_dtype,
+               void *workspace, size_t workspace_bytes, void *stream) {
+  int rc = check_shape(N, R, C, G, dtype);
+  if (rc != GNNHWC_OK) return rc;
+  rc = check_dtypes(dtype, param_dtype, stats_dtype);
+  if (rc != GNNHWC_OK) return rc;
+  if (act < GN_ACT_IDENTITY || act > GN_ACT_GELU_TANH)
+    return fail(GNNHWC_ERR_INVALID_ARGUMENT, "unknown activation code %d", act);
+  if (N == 0 || R == 0) return GNNHWC_OK;  // nothing to normalise; mean / rstd of an empty slab are left untouched
+  if (!x || !y || !mean || !rstd) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "x, y, mean and rstd must not be null");
+  const size_t need = gnnhwc_fwd_workspace_bytes(N, R, C, G, dtype);
+  if (!workspace || !aligned16(workspace) || workspace_bytes < need)
+    return fail(GNNHWC_ERR_WORKSPACE, "forward workspace must be 16-byte aligned and at least %zu bytes (got %p, %zu bytes)",
+                need, workspace, workspace_bytes);
+  const int vec = 16 / elem_size(dtype);
+  const bool vector_ok = C % vec == 0 && aligned16(x) && aligned16(y);
+  FwdArgs a;
+  a.x = x; a.w = weight; a.b = bias; a.y = y; a.mean = mean; a.rstd = rstd;
+  a.eps = eps; a.act = act; a.pdtype = param_dtype; a.sdtype = stats_dtype;
+  a.ws = workspace; a.stream = (hipStream_t)stream;
+  a.plan = make_plan(N, R, C, G, vector_ok ? vec : 1, 1);
+  if (a.plan.nblocks + 64 > 0x7fffffffLL) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "problem needs too many workgroups");
+  hipError_t e;
+  switch (dtype) {
+    case GN_F32: e = launch_fwd_f32(a); break;
+    case GN_F64: e = launch_fwd_f64(a); break;
+    case GN_F16: e = launch_fwd_f16(a); break;
+    default: e = launch_fwd_bf16(a); break;
+  }
+  if (e != hipSuccess) return fail(GNNHWC_ERR_LAUNCH, "forward launch failed: %s", hipGetErrorString(e));
+  return GNNHWC_OK;
+}
+
+int gnnhwc_bwd(const void *dy, const void *x, const void *weight, const void *bias, const void *mean, const void *rstd,
+               void *dx, void *dweight, void *dbias, int64_t N, int64_t R, int64_t C, int64_t G, int act, int dtype,
+               int param_dtype, int stats_dtype, void *workspace, size_t workspace_bytes, void *stream) {
+  int rc = check_shape(N, R, C, G, dtype);
+  if (rc != GNNHWC_OK) return rc;
+  rc = check_dtypes(dtype, param_dtype, stats_dtype);
+  if (rc != GNNHWC_OK) return rc;
+  if (act < GN_ACT_IDENTITY || act > GN_ACT_GELU_TANH)
+    return fail(GNNHWC_ERR_INVALID_ARGUMENT, "unknown activation code %d", act);
+  if (N == 0 || R == 0) {
+    // no elements: the parameter gradients are empty sums
+    const unsigned grid = (unsigned)((C + 255) / 256);
+    if (dweight) hipLaunchKernelGGL(fill_zero_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, dweight, C, param_dtype);
+    if (dbias) hipLaunchKernelGGL(fill_zero_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, dbias, C, param_dtype);
+    const hipError_t e0 = hipGetLastError();
+    if (e0 != hipSuccess) return fail(GNNHWC_ERR_LAUNCH, "backward launch failed: %s", hipGetErrorString(e0));
+    return GNNHWC_OK;
+  }
+  if (!dy || !x || !mean || !rstd || !dx)
+    return fail(GNNHWC_ERR_INVALID_ARGUMENT, "dy, x, mean, rstd and dx must not be null");
+  const size_t need = gnnhwc_bwd_workspace_bytes(N, R, C, G, dtype);
+  if (!workspace || !aligned16(workspace) || workspace_bytes < need)
+    return fail(GNNHWC_ERR_WORKSPACE, "backward workspace must be 16-byte aligned and at least %zu bytes (got %p, %zu bytes)",
+                need, workspace, workspace_bytes);
+  const int vec = 16 / elem_size(dtype);
+  const bool vector_ok = C % vec == 0 && aligned16(x) && aligned16(dy) && aligned16(dx);
+  BwdArgs a;
+  a.dy = dy; a.x = x; a.w = weight; a.b = bias; a.mean = mean; a.rstd = rstd;
+  a.dx = dx; a.dw = dweight; a.db = dbias;
+  a.act = act; a.pdtype = param_dtype; a.sdtype = stats_dtype;
+  a.ws = workspace; a.stream = (hipStream_t)stream;
+  a.plan = make_plan(N, R, C, G, vector_ok ? vec : 1, 2);
+  if (a.plan.nblocks + (C + 255) / 256 + 64 > 0x7fffffffLL)
+    return fail(GNNHWC_ERR_INVALID_ARGUMENT, "problem needs too many workgroups");
+  if (N * G > 0x7fffffffLL) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "N * G too large");
+  hipError_t e;
+  switch (dtype) {
+    case GN_F32: e = launch_bwd_f32(a); break;
+    case GN_F64: e = launch_bwd_f64(a); break;
+    case GN_F16: e = launch_bwd_f16(a); break;
+    default: e = launch_bwd_bf16(a); break;
+  }
+  if (e != hipSuccess) return fail(GNNHWC_ERR_LAUNCH, "backward launch failed: %s", hipGetErrorString(e));
+  return GNNHWC_OK;
+}
+
+int gnnhwc_profile_enable(int on) {
+  g_profile = on != 0;
+  return GNNHWC_OK;
+}
+
+int gnnhwc_profile_collect(int64_t *launches, double *total_ms) {
+  if (!launches || !total_ms) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "null output array");
+  for (int k = 0; k < GNNHWC_NUM_KERNEL_KINDS; ++k) { launches[k] = 0; total_ms[k] = 0.0; }
+  int rc = GNNHWC_OK;
+  for (const Timed &t : g_timed) {
+    float ms = 0.f;
+    hipError_t e = hipEventSynchronize(t.stop);
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, t.start, t.stop);
+    if (e == hipSuccess) {
+      launches[t.kind] += 1;
+      total_ms[t.kind] += ms;
+    } else {
+      rc = fail(GNNHWC_ERR_LAUNCH, "event timing failed: %s", hipGetErrorString(e));
+    }
+    g_event_pool.push_back(t.start);
+    g_event_pool.push_back(t.stop);
+  }
+  g_timed.clear();
+  return rc;
+}
+
+const char *gnnhwc_kernel_kind_name(int kind) {
+  static const char *names[GNNHWC_NUM_KERNEL_KINDS] = {"fwd_stats", "fwd_stats_finalize", "fwd_apply", "bwd_reduce",
+                                                       "bwd_finalize", "bwd_dx", "fused_fwd", "fused_bwd"};
+  return (kind >= 0 && kind < GNNHWC_NUM_KERNEL_KINDS) ? names[kind] : "";
+}
+
+}  // extern "C"

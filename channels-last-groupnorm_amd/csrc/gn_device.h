@@ -1,0 +1,260 @@
+// Device-side building blocks shared by every GroupNorm kernel: element types and 128-bit lane
+// vectors, conversions, activations and their derivatives, and fixed-order reductions.
+// gfx950 (CDNA4) only: wave64, 256 CUs in 8 XCDs.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "gn_plan.h"
+
+namespace gn {
+
+// ---------------------------------------------------------------------------------------------
+// Element types.  Storage types are plain bit containers; all arithmetic is done in the
+// accumulation type (float for f32/f16/bf16, double for f64), with one rounding on store.
+// The reference instead evaluates the half/bfloat16 forward in 16-bit arithmetic
+// (src/gnnhwc/csrc/gn_kernel.cu:294-303); torch's GroupNorm, which defines the expected results,
+// computes in fp32, and so does this code.
+// ---------------------------------------------------------------------------------------------
+struct bf16_t { uint16_t bits; };
+typedef _Float16 f16_t;
+
+template <typename T> struct acc_of { typedef float type; };
+template <> struct acc_of<double> { typedef double type; };
+
+template <typename T> struct vec_of { static constexpr int value = 16 / (int)sizeof(T); };
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef double f64x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t hi16_in_place) {
+  return __builtin_bit_cast(float, hi16_in_place);
+}
+// Round-to-nearest-even float -> bfloat16 pair; clang lowers the fptrunc to v_cvt_pk_bf16_f32 on gfx950.
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  f32x2 f = {lo, hi};
+  bf16x2 b = __builtin_convertvector(f, bf16x2);
+  return __builtin_bit_cast(uint32_t, b);
+}
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
+  __bf16 b = (__bf16)f;
+  return __builtin_bit_cast(uint16_t, b);
+}
+
+// ---- lane vectors: VEC elements of T in one (ideally 128-bit) access ----
+template <typename T, int VEC, bool NT> struct LaneVec;
+
+template <bool NT> struct LaneVec<float, 4, NT> {
+  static __device__ __forceinline__ void load(const float *p, float (&v)[4]) {
+    f32x4 r = NT ? __builtin_nontemporal_load((const f32x4 *)p) : *(const f32x4 *)p;
+    v[0] = r.x; v[1] = r.y; v[2] = r.z; v[3] = r.w;
+  }
+  static __device__ __forceinline__ void store(float *p, const float (&v)[4]) {
+    f32x4 r = {v[0], v[1], v[2], v[3]};
+    if (NT) __builtin_nontemporal_store(r, (f32x4 *)p); else *(f32x4 *)p = r;
+  }
+};
+template <bool NT> struct LaneVec<double, 2, NT> {
+  static __device__ __forceinline__ void load(const double *p, double (&v)[2]) {
+    f64x2 r = NT ? __builtin_nontemporal_load((const f64x2 *)p) : *(const f64x2 *)p;
+    v[0] = r.x; v[1] = r.y;
+  }
+  static __device__ __forceinline__ void store(double *p, const double (&v)[2]) {
+    f64x2 r = {v[0], v[1]};
+    if (NT) __builtin_nontemporal_store(r, (f64x2 *)p); else *(f64x2 *)p = r;
+  }
+};
+template <bool NT> struct LaneVec<f16_t, 8, NT> {
+  static __device__ __forceinline__ void load(const f16_t *p, float (&v)[8]) {
+    f16x8 r = NT ? __builtin_nontemporal_load((const f16x8 *)p) : *(const f16x8 *)p;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = (float)r[j];
+  }
+  static __device__ __forceinline__ void store(f16_t *p, const float (&v)[8]) {
+    f16x8 r;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) r[j] = (_Float16)v[j];  // v_cvt_f16_f32, round to nearest even
+    if (NT) __builtin_nontemporal_store(r, (f16x8 *)p); else *(f16x8 *)p = r;
+  }
+};
+template <bool NT> struct LaneVec<bf16_t, 8, NT> {
+  static __device__ __forceinline__ void load(const bf16_t *p, float (&v)[8]) {
+    u32x4 r = NT ? __builtin_nontemporal_load((const u32x4 *)p) : *(const u32x4 *)p;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      v[2 * j] = bf16_bits_to_float(r[j] << 16);
+      v[2 * j + 1] = bf16_bits_to_float(r[j] & 0xffff0000u);
+    }
+  }
+  static __device__ __forceinline__ void store(bf16_t *p, const float (&v)[8]) {
+    u32x4 r;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r[j] = pack_bf16x2(v[2 * j], v[2 * j + 1]);
+    if (NT) __builtin_nontemporal_store(r, (u32x4 *)p); else *(u32x4 *)p = r;
+  }
+};
+// scalar fall-back: any C, any alignment
+template <bool NT> struct LaneVec<float, 1, NT> {
+  static __device__ __forceinline__ void load(const float *p, float (&v)[1]) { v[0] = *p; }
+  static __device__ __forceinline__ void store(float *p, const float (&v)[1]) { *p = v[0]; }
+};
+template <bool NT> struct LaneVec<double, 1, NT> {
+  static __device__ __forceinline__ void load(const double *p, double (&v)[1]) { v[0] = *p; }
+  static __device__ __forceinline__ void store(double *p, const double (&v)[1]) { *p = v[0]; }
+};
+template <bool NT> struct LaneVec<f16_t, 1, NT> {
+  static __device__ __forceinline__ void load(const f16_t *p, float (&v)[1]) { v[0] = (float)*p; }
+  static __device__ __forceinline__ void store(f16_t *p, const float (&v)[1]) { *p = (_Float16)v[0]; }
+};
+template <bool NT> struct LaneVec<bf16_t, 1, NT> {
+  static __device__ __forceinline__ void load(const bf16_t *p, float (&v)[1]) {
+    v[0] = bf16_bits_to_float((uint32_t)p->bits << 16);
+  }
+  static __device__ __forceinline__ void store(bf16_t *p, const float (&v)[1]) { p->bits = float_to_bf16_bits(v[0]); }
+};
+
+// ---- runtime-typed scalar access to parameters / statistics (read once per workgroup) ----
+template <typename ACC> __device__ __forceinline__ ACC load_scalar(const void *p, int64_t i, int dtype) {
+  switch (dtype) {
+    case GN_F32: return (ACC)((const float *)p)[i];
+    case GN_F64: return (ACC)((const double *)p)[i];
+    case GN_F16: return (ACC)(float)((const _Float16 *)p)[i];
+    default: return (ACC)bf16_bits_to_float((uint32_t)((const uint16_t *)p)[i] << 16);
+  }
+}
+template <typename ACC> __device__ __forceinline__ void store_scalar(void *p, int64_t i, int dtype, ACC v) {
+  switch (dtype) {
+    case GN_F32: ((float *)p)[i] = (float)v; break;
+    case GN_F64: ((double *)p)[i] = (double)v; break;
+    case GN_F16: ((_Float16 *)p)[i] = (_Float16)(float)v; break;
+    default: ((uint16_t *)p)[i] = float_to_bf16_bits((float)v); break;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Activations and derivatives, evaluated in the accumulation type.
+// Definitions follow src/gnnhwc/csrc/gn_kernel.cu:62-106 (identity, relu, silu = x/(1+e^-x),
+// gelu = x/2 (1+erf(x/sqrt2)), gelu_tanh = x/2 (1+tanh(sqrt(2/pi)(x+0.044715x^3)))), which are also
+// the torch definitions (F.relu / F.silu / F.gelu / F.gelu(approximate='tanh')).
+// fp32 forms use the hardware exp2 / rcp (1 ulp each), never a fast-math libm.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+__device__ __forceinline__ double fast_rcp(double x) { return 1.0 / x; }
+// logistic sigmoid 1/(1+e^-x); exp2 overflow to +inf gives rcp(inf) = 0, underflow gives 1.
+__device__ __forceinline__ float sigmoid(float x) {
+  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.44269504088896340736f));
+}
+__device__ __forceinline__ double sigmoid(double x) { return 1.0 / (1.0 + exp(-x)); }
+__device__ __forceinline__ float erf_acc(float x) { return erff(x); }
+__device__ __forceinline__ double erf_acc(double x) { return erf(x); }
+__device__ __forceinline__ float exp_acc(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
+__device__ __forceinline__ double exp_acc(double x) { return exp(x); }
+
+template <int ACT, typename A> __device__ __forceinline__ A act_fwd(A z) {
+  if constexpr (ACT == GN_ACT_IDENTITY) {
+    return z;
+  } else if constexpr (ACT == GN_ACT_RELU) {
+    return z <= (A)0 ? (A)0 : z;  // NaN propagates, like torch.relu
+  } else if constexpr (ACT == GN_ACT_SILU) {
+    return z * sigmoid(z);
+  } else if constexpr (ACT == GN_ACT_GELU) {
+    return (A)0.5 * z * ((A)1 + erf_acc(z * (A)0.70710678118654752440));
+  } else {
+    // 1 + tanh(u) == 2 sigmoid(2u): the same function without the cancellation at u << 0
+    const A u = (A)0.79788456080286535588 * (z + (A)0.044715 * z * z * z);
+    return z * sigmoid((A)2 * u);
+  }
+}
+template <int ACT, typename A> __device__ __forceinline__ A act_bwd(A z) {
+  if constexpr (ACT == GN_ACT_IDENTITY) {
+    return (A)1;
+  } else if constexpr (ACT == GN_ACT_RELU) {
+    return z <= (A)0 ? (A)0 : (A)1;
+  } else if constexpr (ACT == GN_ACT_SILU) {
+    const A s = sigmoid(z);
+    return s * ((A)1 + z * ((A)1 - s));
+  } else if constexpr (ACT == GN_ACT_GELU) {
+    const A cdf = (A)0.5 * ((A)1 + erf_acc(z * (A)0.70710678118654752440));
+    const A pdf = exp_acc((A)-0.5 * z * z) * (A)0.39894228040143267794;
+    return cdf + z * pdf;
+  } else {
+    const A z2 = z * z;
+    const A u = (A)0.79788456080286535588 * (z + (A)0.044715 * z2 * z);
+    const A du = (A)0.79788456080286535588 * ((A)1 + (A)0.134145 * z2);
+    const A s = sigmoid((A)2 * u);  // (1 + tanh u) / 2
+    // d/dz [z s] = s + z * 2 s (1 - s) * du
+    return s + (A)2 * z * s * ((A)1 - s) * du;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Running statistics: (count, mean, M2) triples merged with Chan's parallel update.  Same
+// quantities as WelfordData / WelfordOps::combine (src/gnnhwc/csrc/Welford.h:8-21,44-65); the
+// variance is the biased one, M2 / n (Welford.h:66-72 with correction 0, gn_kernel.cu:175,254).
+// ---------------------------------------------------------------------------------------------
+template <typename A> struct Moments {
+  A n, mean, m2;
+};
+template <typename A> __device__ __forceinline__ Moments<A> merge(const Moments<A> &a, const Moments<A> &b) {
+  const A n = a.n + b.n;
+  if (b.n == (A)0) return a;
+  const A f = b.n * fast_rcp(n);
+  const A d = b.mean - a.mean;
+  Moments<A> r;
+  r.n = n;
+  r.mean = a.mean + d * f;
+  r.m2 = a.m2 + b.m2 + d * d * a.n * f;
+  return r;
+}
+template <typename A> __device__ __forceinline__ A shfl_xor_acc(A v, int mask, int width) {
+  return __shfl_xor(v, mask, width);
+}
+// Butterfly merge over `width` consecutive lanes (power of two <= 64); lane 0 of each segment holds the
+// result of a fixed merge tree, so the outcome does not depend on scheduling.
+template <typename A> __device__ __forceinline__ Moments<A> segment_merge(Moments<A> m, int width) {
+  for (int off = width >> 1; off > 0; off >>= 1) {
+    Moments<A> o;
+    o.n = shfl_xor_acc(m.n, off, width);
+    o.mean = shfl_xor_acc(m.mean, off, width);
+    o.m2 = shfl_xor_acc(m.m2, off, width);
+    // lower lane always merges (self, other), upper lane (other, self): both compute the same value
+    const bool upper = (threadIdx.x & off) != 0;
+    m = upper ? merge(o, m) : merge(m, o);
+  }
+  return m;
+}
+template <typename A> __device__ __forceinline__ A segment_sum(A v, int width) {
+  for (int off = width >> 1; off > 0; off >>= 1) {
+    const A o = shfl_xor_acc(v, off, width);
+    const bool upper = (threadIdx.x & off) != 0;
+    v = upper ? (o + v) : (v + o);
+  }
+  return v;
+}
+
+// Block index -> (sample, row tile, channel chunk).  Blocks are numbered so that consecutive ids
+// (which the hardware deals round-robin to the 8 XCDs) walk the row tiles of one sample; the
+// second pass of a two-pass operation uses `reversed` so that it starts on the tiles the first
+// pass touched last (still in that XCD's L2) while keeping every tile on the same XCD.
+struct TileCoord {
+  int64_t n;
+  int tile, chunk;
+};
+__device__ __forceinline__ TileCoord decode_block(const Plan &p, int64_t b, bool reversed) {
+  if (reversed) {
+    const int64_t full = p.nblocks & ~(int64_t)7;  // blocks in complete octets; the tail keeps its place
+    if (b < full) b = full - 8 - (b & ~(int64_t)7) + (b & 7);
+  }
+  TileCoord t;
+  t.chunk = (int)(b % p.nchunk);
+  const int64_t nt = b / p.nchunk;
+  t.tile = (int)(nt % p.tiles);
+  t.n = nt / p.tiles;
+  return t;
+}
+
+}  // namespace gn

@@ -1,0 +1,35 @@
+// Launch plan shared by host and device code: how an (N, R, C) channels-last slab is cut into
+// workgroup tiles.  Plays the role of the reference's calc_block_params / closest_factor
+// (src/gnnhwc/csrc/gn_kernel.cu:37-60,121-128) but is built around 128-bit lane vectors and
+// 256-thread workgroups instead of <=128-thread blocks over a virtual H x W factorisation.
+#pragma once
+#include <stdint.h>
+
+namespace gn {
+
+enum { GN_F32 = 0, GN_F64 = 1, GN_F16 = 2, GN_BF16 = 3 };
+enum { GN_ACT_IDENTITY = 0, GN_ACT_RELU = 1, GN_ACT_SILU = 2, GN_ACT_GELU = 3, GN_ACT_GELU_TANH = 4 };
+
+constexpr int kBlock = 256;    // threads per workgroup (4 wavefronts)
+constexpr int kUnroll = 4;     // independent row loads in flight per lane
+constexpr int kNumCU = 256;    // MI355X
+constexpr int kTargetBlocks = 2048;  // aim for ~8 workgroups per CU when the tensor is large enough
+
+// One workgroup owns `tile_rows` consecutive rows of one sample and one chunk of `lpr` lane vectors
+// (lpr * vec channels) of every such row.  Inside the workgroup thread t handles lane vector
+// (t % lpr) of rows (t / lpr), (t / lpr) + rpi, ...: every lane keeps the same channels for the whole
+// tile, so per-channel affine coefficients and per-channel partial sums live in registers.
+struct Plan {
+  int64_t N, R, C;
+  int G, D;         // groups, channels per group
+  int vec;          // elements per lane vector (16 bytes / sizeof(T), or 1 for the scalar path)
+  int cv;           // lane vectors per row = C / vec
+  int lpr;          // lane vectors of a row handled by one workgroup (<= kBlock)
+  int nchunk;       // workgroups side by side along C = ceil(cv / lpr)
+  int rpi;          // rows covered per step = kBlock / lpr
+  int tile_rows;    // rows per workgroup tile
+  int tiles;        // row tiles per sample = ceil(R / tile_rows)
+  int64_t nblocks;  // N * tiles * nchunk
+};
+
+}  // namespace gn

@@ -1,0 +1,86 @@
+"""ctypes binding of libgnnhwc_hip.so (C ABI declared in include/gnnhwc.h).
+
+The library is built ahead of time, in-tree, by ``make -C channels-last-groupnorm_amd/csrc`` (or
+``__graft_entry__.build()``).  There is no fallback: if the shared object is missing or does not
+export the expected symbols, importing this module raises.
+"""
+import ctypes
+import os
+
+_CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
+LIB_PATH = os.path.join(_CSRC, "libgnnhwc_hip.so")
+
+# dtype / activation codes of include/gnnhwc.h
+F32, F64, F16, BF16 = 0, 1, 2, 3
+NUM_KERNEL_KINDS = 8
+
+SYMBOLS = (
+    "gnnhwc_version",
+    "gnnhwc_last_error",
+    "gnnhwc_fwd_workspace_bytes",
+    "gnnhwc_bwd_workspace_bytes",
+    "gnnhwc_fwd",
+    "gnnhwc_bwd",
+    "gnnhwc_profile_enable",
+    "gnnhwc_profile_collect",
+    "gnnhwc_kernel_kind_name",
+)
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            "gnnhwc: %s not found. Build the HIP extension first: make -C %s   "
+            "(there is deliberately no non-HIP fallback)" % (LIB_PATH, _CSRC)
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    i64, vp, ci, sz, dbl = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_double
+    for name in SYMBOLS:
+        if not hasattr(lib, name):
+            raise ImportError("gnnhwc: %s does not export %s" % (LIB_PATH, name))
+    lib.gnnhwc_version.restype = ci
+    lib.gnnhwc_last_error.restype = ctypes.c_char_p
+    lib.gnnhwc_fwd_workspace_bytes.argtypes = [i64, i64, i64, i64, ci]
+    lib.gnnhwc_fwd_workspace_bytes.restype = sz
+    lib.gnnhwc_bwd_workspace_bytes.argtypes = [i64, i64, i64, i64, ci]
+    lib.gnnhwc_bwd_workspace_bytes.restype = sz
+    lib.gnnhwc_fwd.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, dbl, ci, ci, ci, ci, vp, sz, vp]
+    lib.gnnhwc_fwd.restype = ci
+    lib.gnnhwc_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, ci, ci, ci, ci, vp, sz, vp]
+    lib.gnnhwc_bwd.restype = ci
+    lib.gnnhwc_profile_enable.argtypes = [ci]
+    lib.gnnhwc_profile_enable.restype = ci
+    lib.gnnhwc_profile_collect.argtypes = [ctypes.POINTER(i64), ctypes.POINTER(dbl)]
+    lib.gnnhwc_profile_collect.restype = ci
+    lib.gnnhwc_kernel_kind_name.argtypes = [ci]
+    lib.gnnhwc_kernel_kind_name.restype = ctypes.c_char_p
+    return lib
+
+
+lib = _load()
+
+
+def last_error():
+    return lib.gnnhwc_last_error().decode("utf-8", "replace")
+
+
+def check(rc, what):
+    if rc != 0:
+        raise RuntimeError("%s failed (code %d): %s" % (what, rc, last_error()))
+
+
+def kernel_kind_names():
+    return [lib.gnnhwc_kernel_kind_name(k).decode() for k in range(NUM_KERNEL_KINDS)]
+
+
+def profile_enable(on):
+    check(lib.gnnhwc_profile_enable(1 if on else 0), "gnnhwc_profile_enable")
+
+
+def profile_collect():
+    """Returns {kind name: (launches, total milliseconds)} since the previous collect."""
+    n = (ctypes.c_int64 * NUM_KERNEL_KINDS)()
+    ms = (ctypes.c_double * NUM_KERNEL_KINDS)()
+    check(lib.gnnhwc_profile_collect(n, ms), "gnnhwc_profile_collect")
+    names = kernel_kind_names()
+    return {names[k]: (int(n[k]), float(ms[k])) for k in range(NUM_KERNEL_KINDS)}

@@ -1,0 +1,214 @@
+"""Python surface of the NHWC GroupNorm op: ``GN_NHWC`` (an ``nn.GroupNorm`` subclass with a fused
+activation), its ``autograd.Function`` and the ``gnop::fwd`` / ``gnop::bwd`` operators.
+
+Mirrors src/gnnhwc/custom_gn.py:29-90 and the operator glue src/gnnhwc/csrc/custom_gn.cpp:10-94 of the
+reference; the kernels behind the operators are the HIP ones in libgnnhwc_hip.so, reached through its
+C ABI (include/gnnhwc.h) with raw device pointers and the current HIP stream.  torch only provides
+device memory (outputs, workspace) and the stream.
+"""
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import _cabi
+
+_DTYPE_CODE = {
+    torch.float32: _cabi.F32,
+    torch.float64: _cabi.F64,
+    torch.float16: _cabi.F16,
+    torch.bfloat16: _cabi.BF16,
+}
+
+# custom_gn.py:52-59
+ACTIVATION_CODES = {
+    "identity": 0,
+    "relu": 1,
+    "swish": 2,
+    "silu": 2,
+    "gelu": 3,
+    "gelu_tanh": 4,
+}
+
+
+def _check_device(t, name):
+    # CHECK_CUDA, custom_gn.cpp:8,17-19,53-58 (a ROCm build of torch calls the HIP device "cuda")
+    if not t.is_cuda:
+        raise RuntimeError("%s must be a CUDA tensor" % name)
+
+
+def _dtype_code(t, name):
+    try:
+        return _DTYPE_CODE[t.dtype]
+    except KeyError:
+        # AT_DISPATCH_FLOATING_TYPES_AND2 raises for any other type (custom_gn.cpp:29-33)
+        raise RuntimeError('"group_norm_nhwc" not implemented for %s (%s)' % (t.dtype, name)) from None
+
+
+def _stats_dtype(x_dtype):
+    # The reference allocates mean / rstd in the parameters' (= data's) dtype (custom_gn.cpp:26-27).
+    # For 16-bit data that rounding would leak into dx, so statistics are kept in float32 there.
+    return torch.float32 if x_dtype in (torch.float16, torch.bfloat16) else x_dtype
+
+
+def _as_nrc(t):
+    """(N, C, R) tensor with strides (R*C, 1, C) -> contiguous (N, R, C) view (copies only if it must)."""
+    t = t.permute(0, 2, 1)
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def _workspace(nbytes, device):
+    return torch.empty((nbytes,), dtype=torch.uint8, device=device)
+
+
+def gn_nhwc_fwd(X, weight, bias, G, eps, act_fn_option):
+    """gnop::fwd -- custom_gn.cpp:10-42.  X: (N, C, R) channels-last view.  Returns (Y, means, rstds)."""
+    _check_device(X, "X")
+    _check_device(weight, "weight")
+    _check_device(bias, "bias")
+    if X.dim() != 3:
+        raise RuntimeError("gnop::fwd expects X of shape (N, C, R), got %s" % (tuple(X.shape),))
+    N, C, R = X.shape
+    dt = _dtype_code(X, "X")
+    pdt = _dtype_code(weight, "weight")
+    if bias.dtype != weight.dtype:
+        raise RuntimeError("weight and bias must have the same dtype (%s vs %s)" % (weight.dtype, bias.dtype))
+    if weight.numel() != C or bias.numel() != C:
+        raise RuntimeError("weight and bias must have %d elements" % C)
+    X_nrc = _as_nrc(X)
+    Y = torch.empty_like(X_nrc)
+    sdtype = _stats_dtype(X.dtype)
+    means = torch.empty((N, G), dtype=sdtype, device=X.device)
+    rstds = torch.empty((N, G), dtype=sdtype, device=X.device)
+    lib = _cabi.lib
+    with torch.cuda.device(X.device):
+        nbytes = lib.gnnhwc_fwd_workspace_bytes(N, R, C, G, dt)
+        if nbytes == 0:
+            raise RuntimeError("gnop::fwd: " + _cabi.last_error())
+        ws = _workspace(nbytes, X.device)
+        rc = lib.gnnhwc_fwd(
+            X_nrc.data_ptr(), weight.contiguous().data_ptr(), bias.contiguous().data_ptr(),
+            Y.data_ptr(), means.data_ptr(), rstds.data_ptr(),
+            N, R, C, G, float(eps), int(act_fn_option), dt, pdt, _DTYPE_CODE[sdtype],
+            ws.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream)
+    _cabi.check(rc, "gnop::fwd")
+    return Y.permute(0, 2, 1), means, rstds
+
+
+def gn_nhwc_bwd(dy, X, weight, bias, means, rstds, G, act_fn_option):
+    """gnop::bwd -- custom_gn.cpp:44-89.  Returns (dX (N, C, R) channels-last view, dweight, dbias)."""
+    for t, name in ((dy, "dy"), (X, "X"), (weight, "weight"), (bias, "bias"), (means, "means"), (rstds, "rstds")):
+        _check_device(t, name)
+    if X.dim() != 3 or dy.shape != X.shape:
+        raise RuntimeError("gnop::bwd expects dy and X of the same shape (N, C, R), got %s and %s"
+                           % (tuple(dy.shape), tuple(X.shape)))
+    N, C, R = X.shape
+    dt = _dtype_code(X, "X")
+    pdt = _dtype_code(weight, "weight")
+    sdt = _dtype_code(means, "means")
+    if dy.dtype != X.dtype:
+        raise RuntimeError("dy and X must have the same dtype (%s vs %s)" % (dy.dtype, X.dtype))
+    if rstds.dtype != means.dtype or bias.dtype != weight.dtype:
+        raise RuntimeError("means/rstds and weight/bias must pairwise share a dtype")
+    if means.numel() != N * G or rstds.numel() != N * G:
+        raise RuntimeError("means and rstds must have N*G = %d elements" % (N * G))
+    X_nrc = _as_nrc(X)
+    dy_nrc = _as_nrc(dy)
+    dX = torch.empty_like(X_nrc)
+    dweight = torch.empty((C,), dtype=weight.dtype, device=X.device)
+    dbias = torch.empty((C,), dtype=weight.dtype, device=X.device)
+    lib = _cabi.lib
+    with torch.cuda.device(X.device):
+        nbytes = lib.gnnhwc_bwd_workspace_bytes(N, R, C, G, dt)
+        if nbytes == 0:
+            raise RuntimeError("gnop::bwd: " + _cabi.last_error())
+        ws = _workspace(nbytes, X.device)
+        rc = lib.gnnhwc_bwd(
+            dy_nrc.data_ptr(), X_nrc.data_ptr(), weight.contiguous().data_ptr(), bias.contiguous().data_ptr(),
+            means.contiguous().data_ptr(), rstds.contiguous().data_ptr(),
+            dX.data_ptr(), dweight.data_ptr(), dbias.data_ptr(),
+            N, R, C, G, int(act_fn_option), dt, pdt, sdt,
+            ws.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream)
+    _cabi.check(rc, "gnop::bwd")
+    return dX.permute(0, 2, 1), dweight, dbias
+
+
+# TORCH_LIBRARY(gnop, m) { m.def("fwd", ...); m.def("bwd", ...); } -- custom_gn.cpp:91-94.  The reference
+# registers catch-all kernels that themselves reject non-device tensors; CompositeExplicitAutograd plays that
+# role here, so a CPU tensor reaches the "must be a CUDA tensor" check instead of a dispatcher error.
+_op_lib = torch.library.Library("gnop", "DEF")
+_op_lib.define("fwd(Tensor X, Tensor weight, Tensor bias, int G, float eps, int act_fn_option) -> (Tensor, Tensor, Tensor)")
+_op_lib.define("bwd(Tensor dy, Tensor X, Tensor weight, Tensor bias, Tensor means, Tensor rstds, int G, "
+               "int act_fn_option) -> (Tensor, Tensor, Tensor)")
+_op_lib.impl("fwd", gn_nhwc_fwd, "CompositeExplicitAutograd")
+_op_lib.impl("bwd", gn_nhwc_bwd, "CompositeExplicitAutograd")
+
+
+class GN_NHWC_Func(torch.autograd.Function):
+    """custom_gn.py:29-47.  apply(X, weight, bias, G, eps, activation_code) -> Y with X's shape and strides."""
+
+    @staticmethod
+    def forward(ctx, X, weight, bias, G, eps, activation):
+        ctx.x_shape = X.shape
+        X_flat = X.view(X.shape[0], X.shape[1], -1)
+        X_out, means, rstds = torch.ops.gnop.fwd(X_flat, weight, bias, G, eps, activation)
+        ctx.save_for_backward(X_flat, weight, bias, means, rstds)
+        ctx.G = G
+        ctx.activation = activation
+        return X_out.view(ctx.x_shape)
+
+    @staticmethod
+    def backward(ctx, dy):
+        X_flat, weight, bias, means, rstds = ctx.saved_tensors
+        # Bring dy into X's own layout (channels fastest, spatial dims in X's order).  The reference uses
+        # dy.contiguous(memory_format=channels_last) (custom_gn.py:44), which only exists for 4-D tensors;
+        # permuting the channel axis to the end and back works for any rank >= 3.
+        nd = dy.dim()
+        dy_last = dy.permute(0, *range(2, nd), 1).contiguous()
+        dy_flat = dy_last.view(dy_last.shape[0], -1, dy_last.shape[-1]).permute(0, 2, 1)
+        assert dy_flat.stride() == X_flat.stride() or X_flat.numel() == 0 or 1 in X_flat.shape
+        dx, dgamma, dbeta = torch.ops.gnop.bwd(dy_flat, X_flat, weight, bias, means, rstds, ctx.G, ctx.activation)
+        return dx.view(ctx.x_shape), dgamma, dbeta, None, None, None
+
+
+_TORCH_ACTIVATIONS = (
+    lambda t: t,
+    F.relu,
+    F.silu,
+    F.gelu,
+    lambda t: F.gelu(t, approximate="tanh"),
+)
+
+
+class GN_NHWC(nn.GroupNorm):
+    """custom_gn.py:49-90.  GroupNorm over channels-last input with the activation applied in the same pass."""
+
+    def __init__(self, num_groups, num_channels, activation="identity", **kwargs):
+        super().__init__(num_groups, num_channels, **kwargs)
+        self.activation = activation
+        self.act_code = ACTIVATION_CODES[activation]  # unknown name -> KeyError, as in the reference
+
+    @torch._dynamo.disable
+    def forward(self, x):
+        if x.stride(1) == 1:
+            # channels fastest.  Make the remaining dims contiguous in their logical order as well: a shape
+            # (2, 3, 5, 9) input must have strides (135, 1, 27, 3), not e.g. (135, 1, 3, 15) (custom_gn.py:68-73).
+            nd = x.dim()
+            x = x.permute(0, *range(2, nd), 1).contiguous().permute(0, nd - 1, *range(1, nd - 1))
+            run = GN_NHWC_Func.apply
+        else:
+            # channels-first input: torch's own GroupNorm, then the activation (custom_gn.py:75-79)
+            x = x.contiguous()
+            act = _TORCH_ACTIVATIONS[self.act_code]
+
+            def run(t, w, b, g, eps, _code):
+                return act(F.group_norm(t, g, w, b, eps))
+
+        if self.affine:
+            w, b = self.weight, self.bias
+        else:  # custom_gn.py:83-86
+            w = torch.ones((self.num_channels,), device=x.device, dtype=x.dtype)
+            b = torch.zeros((self.num_channels,), device=x.device, dtype=x.dtype)
+        return run(x, w, b, self.num_groups, self.eps, self.act_code)
+
+    def extra_repr(self):
+        return "{num_groups}, {num_channels}, eps={eps}, affine={affine}, activation={activation}".format(**self.__dict__)

@@ -1,0 +1,124 @@
+/*
+ * gnnhwc.h -- C ABI of libgnnhwc_hip.so: channels-last (NHWC) GroupNorm forward / backward
+ * with a fused activation, for AMD gfx950 (MI355X).
+ *
+ * This is the drop-in boundary for the reference's raw kernel interface
+ *   run_gn_fwd_kernels<T> / run_gn_bwd_kernels<T>   (src/gnnhwc/csrc/gn_kernel.h:11-41)
+ * which its op glue calls from gn_nhwc_fwd / gn_nhwc_bwd (src/gnnhwc/csrc/custom_gn.cpp:10-89).
+ * The template parameter T becomes a runtime dtype code, `int` sizes become int64_t, the implicit
+ * "current CUDA stream" becomes an explicit hipStream_t, and the scratch memory the reference takes
+ * from the caching allocator inside the host driver (gn_kernel.cu:461,954-1001) becomes a
+ * caller-provided workspace whose size is queried up front.  No torch types appear here.
+ *
+ * Tensor layout (identical to the reference's permuted views, custom_gn.cpp:24,64-65):
+ *   x, y, dy, dx : (N, R, C) contiguous, C fastest; R = product of all spatial dims.
+ *   weight, bias, dweight, dbias : (C) in `param_dtype`; weight/bias may be NULL (gamma=1, beta=0).
+ *   mean, rstd   : (N, G) in `stats_dtype`.
+ * All pointers are device pointers on the device that is current for the calling thread.
+ * Calls are asynchronous on `stream` and never synchronise; the library is stateless apart from a
+ * per-thread error string, so concurrent calls on different streams are safe as long as each call
+ * has its own workspace.
+ *
+ * Every entry point returns GNNHWC_OK (0) or a negative error code; gnnhwc_last_error() describes the
+ * most recent failure on the calling thread.  Nothing is launched when an error is returned.
+ */
+#ifndef GNNHWC_H
+#define GNNHWC_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* dtype codes -- the four types of AT_DISPATCH_FLOATING_TYPES_AND2(Half, BFloat16, ...)
+ * (custom_gn.cpp:29-33, 73-77). */
+enum {
+  GNNHWC_F32 = 0,
+  GNNHWC_F64 = 1,
+  GNNHWC_F16 = 2,
+  GNNHWC_BF16 = 3
+};
+
+/* activation codes -- same integers as GN_NHWC.act_code (custom_gn.py:52-59) and the
+ * act_fn_option switch of the reference host drivers (gn_kernel.cu:419-436, 911-929). */
+enum {
+  GNNHWC_ACT_IDENTITY = 0,
+  GNNHWC_ACT_RELU = 1,
+  GNNHWC_ACT_SILU = 2,
+  GNNHWC_ACT_GELU = 3,
+  GNNHWC_ACT_GELU_TANH = 4
+};
+
+enum {
+  GNNHWC_OK = 0,
+  GNNHWC_ERR_INVALID_ARGUMENT = -1, /* bad shape / dtype / activation / null pointer          */
+  GNNHWC_ERR_WORKSPACE = -2,        /* workspace null, misaligned or smaller than required     */
+  GNNHWC_ERR_LAUNCH = -3            /* the HIP runtime rejected a launch (message has details) */
+};
+
+/* Library version, (major << 16) | minor. */
+int gnnhwc_version(void);
+
+/* Human-readable description of the last error on this thread ("" if none). */
+const char *gnnhwc_last_error(void);
+
+/*
+ * Bytes of device workspace gnnhwc_fwd / gnnhwc_bwd need for this problem (0 is never returned
+ * for a valid shape; returns 0 and sets the error string for an invalid one).  The workspace must
+ * be 256-byte aligned; its contents on entry are ignored and are undefined on return.
+ * Replaces: raw_alloc of the Welford scratch (gn_kernel.cu:461) and of the seven backward
+ * scratch buffers (gn_kernel.cu:954,973-974,998-1001).
+ */
+size_t gnnhwc_fwd_workspace_bytes(int64_t N, int64_t R, int64_t C, int64_t G, int dtype);
+size_t gnnhwc_bwd_workspace_bytes(int64_t N, int64_t R, int64_t C, int64_t G, int dtype);
+
+/*
+ * Forward: per-(n, group) mean / rstd = 1/sqrt(var + eps) (biased variance), then
+ *   y = act((x - mean) * rstd * weight + bias).
+ * Replaces run_gn_fwd_kernels<T> (gn_kernel.h:11-24; gn_kernel.cu:439-531).
+ *   dtype        : type of x and y.
+ *   param_dtype  : type of weight and bias (the reference requires it to equal dtype,
+ *                  custom_gn.cpp:35; here GNNHWC_F32 parameters with F16/BF16 data are also accepted).
+ *   stats_dtype  : type mean / rstd are written in; equal to dtype, or GNNHWC_F32 for F16/BF16 data.
+ * Statistics are always accumulated and applied in fp32 (fp64 for F64) whatever stats_dtype is.
+ */
+int gnnhwc_fwd(const void *x, const void *weight, const void *bias,
+               void *y, void *mean, void *rstd,
+               int64_t N, int64_t R, int64_t C, int64_t G,
+               double eps, int act,
+               int dtype, int param_dtype, int stats_dtype,
+               void *workspace, size_t workspace_bytes, void *stream /* hipStream_t */);
+
+/*
+ * Backward: given dy and the forward's inputs and statistics, recomputes the activation gradient and
+ * returns dx (N,R,C), dweight (C) and dbias (C).
+ * Replaces run_gn_bwd_kernels<T> (gn_kernel.h:26-41; gn_kernel.cu:932-1055).
+ *   dweight / dbias are written in param_dtype; either may be NULL to skip it.
+ */
+int gnnhwc_bwd(const void *dy, const void *x, const void *weight, const void *bias,
+               const void *mean, const void *rstd,
+               void *dx, void *dweight, void *dbias,
+               int64_t N, int64_t R, int64_t C, int64_t G, int act,
+               int dtype, int param_dtype, int stats_dtype,
+               void *workspace, size_t workspace_bytes, void *stream /* hipStream_t */);
+
+/*
+ * Per-kernel timing for benchmarks (no counterpart in the reference, which relies on an external
+ * profiler, prof.py:1-39).  While enabled, every kernel the library launches on this thread is
+ * bracketed by HIP events on the launch stream.  gnnhwc_profile_collect synchronises those events and
+ * reports, for each kernel kind, the number of launches and the summed duration in milliseconds since
+ * the last collect, then clears the record.  Kinds: 0 fwd statistics, 1 fwd statistics finalize,
+ * 2 fwd apply, 3 bwd reduce, 4 bwd finalize, 5 bwd dx, 6 fused single-kernel fwd, 7 fused single-kernel bwd.
+ */
+#define GNNHWC_NUM_KERNEL_KINDS 8
+int gnnhwc_profile_enable(int on);
+int gnnhwc_profile_collect(int64_t *launches /* [GNNHWC_NUM_KERNEL_KINDS] */,
+                           double *total_ms /* [GNNHWC_NUM_KERNEL_KINDS] */);
+const char *gnnhwc_kernel_kind_name(int kind);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GNNHWC_H */
