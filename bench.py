@@ -1,0 +1,337 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused NHWC GroupNorm + activation forward / backward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload sd_unet|<config name>] [--all]
+
+A "step" is one forward + backward call of the op, through the C ABI of libgnnhwc_hip.so, on each shape
+of the workload (default: the latent-diffusion UNet sweep c3a, c3b, c3c in bf16 with fused SiLU), with
+inputs, outputs and workspaces already resident in HBM.  The timed region is K steps between two
+torch.cuda.synchronize() calls.  Prints ONE JSON line:
+
+  value        algorithmic GB/s of the timed region: (2 S fwd + 3 S bwd per shape) / time
+  roofline     the dominant kernel's algorithmic bytes per launch / its mean duration, measured here with
+               HIP events recorded on the launch stream around every launch, against 8 TB/s
+  cpu_baseline torch.nn.functional.group_norm + SiLU + autograd on the host cores, same tensors (bounded sample)
+  shapes       per-shape us/call and GB/s, with warm (same buffers every call) and cold (rotating through
+               > 512 MB of distinct buffers) figures
+"""
+import argparse
+import ctypes
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "channels-last-groupnorm_amd"))
+
+HBM_PEAK_GBPS = 8000.0
+# algorithmic bytes of each kernel kind, in units of S = bytes of one activation-sized tensor
+KERNEL_STREAMS = {"fwd_stats": 1, "fwd_stats_finalize": 0, "fwd_apply": 2, "bwd_reduce": 2, "bwd_finalize": 0, "bwd_dx": 3,
+                  "fused_fwd": 2, "fused_bwd": 3}
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="sd_unet")
+    ap.add_argument("--all", action="store_true", help="also time every other configuration (reported under 'shapes')")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a replayed HIP graph")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
+    return ap.parse_args()
+
+
+class Problem:
+    """Device buffers for one configuration: `nsets` independent sets of x, dy, y, dx (+ shared parameters)."""
+
+    def __init__(self, cfg, device, nsets=1):
+        import torch
+        from tests import configs
+        from tests.gpu_harness import nrc_view
+
+        self.cfg = cfg
+        self.S = configs.tensor_bytes(cfg)
+        inp = configs.make_inputs(cfg, device)
+        x, dy = nrc_view(inp["x"]), nrc_view(inp["dy"])
+        self.N, self.R, self.C = x.shape
+        self.G = cfg.G
+        from oracle.gn_oracle import ACT_CODES  # name -> code table only
+
+        self.act = ACT_CODES[cfg.act]
+        self.w, self.b = inp["w"], inp["b"]
+        self.sets = []
+        for i in range(nsets):
+            xs = x if i == 0 else x.clone()
+            dys = dy if i == 0 else dy.clone()
+            self.sets.append(dict(x=xs, dy=dys, y=torch.empty_like(xs), dx=torch.empty_like(xs)))
+        sd = torch.float32 if x.dtype in (torch.float16, torch.bfloat16) else x.dtype
+        self.mean = torch.empty((self.N, self.G), dtype=sd, device=device)
+        self.rstd = torch.empty((self.N, self.G), dtype=sd, device=device)
+        self.dw = torch.empty((self.C,), dtype=self.w.dtype, device=device)
+        self.db = torch.empty((self.C,), dtype=self.w.dtype, device=device)
+        from gnnhwc import _cabi
+        from tests.gpu_harness import DT_CODE
+
+        self.lib = _cabi.lib
+        self.dt = DT_CODE[x.dtype]
+        self.sdt = DT_CODE[sd]
+        fb = self.lib.gnnhwc_fwd_workspace_bytes(self.N, self.R, self.C, self.G, self.dt)
+        bb = self.lib.gnnhwc_bwd_workspace_bytes(self.N, self.R, self.C, self.G, self.dt)
+        self.ws_f = torch.empty((fb,), dtype=torch.uint8, device=device)
+        self.ws_b = torch.empty((bb,), dtype=torch.uint8, device=device)
+        self.bwd = cfg.passes != "fwd"
+
+    def alg_bytes(self):
+        return (5 if self.bwd else 2) * self.S
+
+    def fwd(self, s, stream):
+        b = self.sets[s]
+        rc = self.lib.gnnhwc_fwd(b["x"].data_ptr(), self.w.data_ptr(), self.b.data_ptr(), b["y"].data_ptr(),
+                                 self.mean.data_ptr(), self.rstd.data_ptr(), self.N, self.R, self.C, self.G, 1e-5, self.act,
+                                 self.dt, self.dt, self.sdt, self.ws_f.data_ptr(), self.ws_f.numel(), stream)
+        if rc != 0:
+            raise RuntimeError(self.lib.gnnhwc_last_error().decode())
+
+    def bwd_(self, s, stream):
+        b = self.sets[s]
+        rc = self.lib.gnnhwc_bwd(b["dy"].data_ptr(), b["x"].data_ptr(), self.w.data_ptr(), self.b.data_ptr(),
+                                 self.mean.data_ptr(), self.rstd.data_ptr(), b["dx"].data_ptr(), self.dw.data_ptr(),
+                                 self.db.data_ptr(), self.N, self.R, self.C, self.G, self.act, self.dt, self.dt, self.sdt,
+                                 self.ws_b.data_ptr(), self.ws_b.numel(), stream)
+        if rc != 0:
+            raise RuntimeError(self.lib.gnnhwc_last_error().decode())
+
+    def step(self, s, stream, which="both"):
+        if which in ("both", "fwd"):
+            self.fwd(s, stream)
+        if self.bwd and which in ("both", "bwd"):
+            self.bwd_(s, stream)
+
+
+def time_region(fn_step, steps, warmup, use_graph, reps=1):
+    """Time `steps` calls of fn_step() between two device synchronisations; returns seconds (median of reps).
+    With use_graph the K calls are captured once into a HIP graph and the graph is replayed."""
+    import torch
+
+    if use_graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(max(3, min(warmup, 5))):
+                fn_step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(steps):
+                fn_step()
+        run = g.replay
+        nwarm = max(1, warmup // max(1, steps) + 1)
+    else:
+        def run():
+            for _ in range(steps):
+                fn_step()
+        nwarm = 1
+        for _ in range(warmup):
+            fn_step()
+    for _ in range(nwarm):
+        run()
+    times = []
+    for _ in range(reps):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        run()
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+    return statistics.median(times)
+
+
+def measure_shape(prob_warm, prob_cold, steps, warmup, use_graph):
+    """us/call and GB/s for one configuration: fwd, bwd and fwd+bwd; warm and cold."""
+    import torch
+
+    out = {}
+    for label, prob in (("warm", prob_warm), ("cold", prob_cold)):
+        if prob is None:
+            continue
+        nsets = len(prob.sets)
+        for which in (("fwd", "bwd", "both") if prob.bwd else ("fwd",)):
+            ctr = [0]
+
+            def one():
+                stream = torch.cuda.current_stream().cuda_stream
+                prob.step(ctr[0] % nsets, stream, which)
+                ctr[0] += 1
+
+            k = steps if label == "warm" else max(nsets, (steps // nsets) * nsets)
+            ctr[0] = 0
+            t = time_region(one, k, warmup, use_graph, reps=5)
+            us = t / k * 1e6
+            nbytes = {"fwd": 2, "bwd": 3, "both": 5 if prob.bwd else 2}[which] * prob.S
+            key = {"fwd": "fwd", "bwd": "bwd", "both": "fwd_bwd"}[which] if prob.bwd else "fwd"
+            out["%s_%s_us" % (label, key)] = round(us, 3)
+            out["%s_%s_gbps" % (label, key)] = round(nbytes / (t / k) / 1e9, 1)
+    return out
+
+
+def kernel_profile(probs, steps):
+    """Mean duration of every kernel kind over `steps` eager steps, from HIP events around each launch."""
+    import torch
+    from gnnhwc import _cabi
+
+    stream = torch.cuda.current_stream().cuda_stream
+    torch.cuda.synchronize()
+    _cabi.profile_enable(True)
+    try:
+        for _ in range(steps):
+            for p in probs:
+                p.step(0, stream)
+        res = _cabi.profile_collect()
+    finally:
+        _cabi.profile_enable(False)
+    return res
+
+
+def cpu_baseline(cfg_names, seconds):
+    """torch's CPU GroupNorm + activation + autograd on the host cores, same seeded tensors and dtype."""
+    import torch
+    from oracle import gn_oracle as orc  # the checker's torch_reference: the CPU baseline leg
+    from tests import configs
+
+    per = {}
+    total_bytes, total_time = 0.0, 0.0
+    budget = seconds / len(cfg_names)
+    for name in cfg_names:
+        cfg = configs.CONFIGS[name]
+        inp = configs.make_inputs(cfg, "cpu")
+        dy = inp["dy"] if cfg.passes != "fwd" else None
+        ts = []
+        t_begin = time.perf_counter()
+        n = 0
+        while n < 3 or (n < 13 and time.perf_counter() - t_begin < budget):
+            t0 = time.perf_counter()
+            orc.torch_reference(inp["x"], inp["w"], inp["b"], cfg.G, 1e-5, cfg.act, dy)
+            ts.append(time.perf_counter() - t0)
+            n += 1
+        ts = ts[1:] if len(ts) > 3 else ts  # first call pays one-off set-up
+        med = statistics.median(ts)
+        per[name] = round(med * 1e6, 1)
+        total_bytes += configs.algorithmic_bytes(cfg)
+        total_time += med
+    return {
+        "value": round(total_bytes / total_time / 1e9, 3),
+        "unit": "GB/s",
+        "cores": torch.get_num_threads(),
+        "host_cpus": os.cpu_count(),
+        "kind": "port",
+        "sample": "torch.nn.functional.group_norm + activation + autograd.grad on CPU (the results contract), same seeded "
+                  "tensors and dtype, median of up to 12 calls per shape after 1 discarded; us/call per shape: %s" % json.dumps(per),
+        "us_per_call": per,
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (GroupNorm statistics are per sample; nothing is exchanged "
+              "between GPUs). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from tests import configs
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    use_graph = not args.no_graph
+
+    head_names = list(configs.SD_UNET_SWEEP) if args.workload == "sd_unet" else [args.workload]
+    probs = [Problem(configs.CONFIGS[n], device) for n in head_names]
+    stream_of = lambda: torch.cuda.current_stream().cuda_stream  # noqa: E731
+
+    def step():
+        s = stream_of()
+        for p in probs:
+            p.step(0, s)
+
+    # ---- headline: K steps between synchronisations ----
+    t = time_region(step, args.steps, args.warmup, use_graph, reps=1)
+    alg = sum(p.alg_bytes() for p in probs)
+    ms_per_step = t / args.steps * 1e3
+    value = alg / (t / args.steps) / 1e9
+    t_eager = time_region(step, args.steps, args.warmup, False, reps=1)
+
+    # ---- per-kernel durations (HIP events on the launch stream) ----
+    prof = kernel_profile(probs, max(20, args.steps // 4))
+    kinds = {k: v for k, v in prof.items() if v[0] > 0}
+    dominant = max(kinds, key=lambda k: kinds[k][1])
+    launches, total_ms = kinds[dominant]
+    mean_S = sum(p.S for p in probs) / len(probs)
+    achieved = KERNEL_STREAMS[dominant] * mean_S / (total_ms / launches * 1e-3) / 1e9
+    roofline = {
+        "bound": "hbm",
+        "kernel": dominant,
+        "achieved": round(achieved, 1),
+        "peak": HBM_PEAK_GBPS,
+        "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBPS, 4),
+        "traffic": None,
+        "bytes_per_launch": KERNEL_STREAMS[dominant] * mean_S,
+        "mean_launch_us": round(total_ms / launches * 1e3, 3),
+        "kernels_us": {k: round(v[1] / v[0] * 1e3, 3) for k, v in kinds.items()},
+    }
+
+    # ---- per-shape table ----
+    shapes = {}
+    names = list(configs.ALL_NAMES) if args.all else head_names
+    for n in names:
+        cfg = configs.CONFIGS[n]
+        S = configs.tensor_bytes(cfg)
+        nsets = max(2, int(600e6 // (4 * S)) + 1)
+        warm = Problem(cfg, device, 1)
+        cold = Problem(cfg, device, nsets)
+        k = max(20, args.steps // 2)
+        r = measure_shape(warm, cold, k, args.warmup, use_graph)
+        r.update(dtype=cfg.dtype, shape=list(cfg.shape), G=cfg.G, act=cfg.act, S_bytes=S)
+        key = "fwd_bwd" if cfg.passes != "fwd" else "fwd"
+        r["warm_frac_of_peak"] = round(r["warm_%s_gbps" % key] / HBM_PEAK_GBPS, 4)
+        r["cold_frac_of_peak"] = round(r["cold_%s_gbps" % key] / HBM_PEAK_GBPS, 4)
+        shapes[n] = r
+        del warm, cold
+        torch.cuda.empty_cache()
+
+    line = {
+        "metric": "fused GN+SiLU fwd+bwd achieved HBM GB/s (algorithmic bytes / time), SD-UNet shapes",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "us_per_call": {p.cfg.name: shapes[p.cfg.name].get("warm_fwd_bwd_us", shapes[p.cfg.name].get("warm_fwd_us")) for p in probs},
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": {"bf16": "bf16 data, f32 arithmetic", "fp16": "f16 data, f32 arithmetic", "fp32": "f32", "fp64": "f64"}[probs[0].cfg.dtype],
+        "data": "synthetic (seeded)",
+        "config": {"workload": "+".join(head_names), "passes": "fwd+bwd", "activation": probs[0].cfg.act,
+                   "timing": "HIP graph replay of the K steps" if use_graph else "eager launches",
+                   "algorithmic_bytes_per_step": alg},
+        "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
+        "eager_ms_per_step": round(t_eager / args.steps * 1e3, 5),
+        "roofline": roofline,
+        "shapes": shapes,
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(head_names, args.cpu_seconds)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -67,7 +67,7 @@ Plan make_plan(int64_t N, int64_t R, int64_t C, int64_t G, int vec, int streams)
   if (forced_lpr > 0 && forced_lpr <= kBlock && forced_lpr <= p.cv) {
     lpr = forced_lpr;
   } else if (vec > 1) {
-    static const int preferred[] = {16, 32, 8, 64, 128, 256};
+    static const int preferred[] = {8, 16, 32, 64, 128, 256};
     for (int d : preferred)
       if (p.cv % d == 0) { lpr = d; break; }
   }
@@ -81,23 +81,30 @@ Plan make_plan(int64_t N, int64_t R, int64_t C, int64_t G, int vec, int streams)
   const int64_t lane_rows = (R + p.rpi - 1) / p.rpi;  // steps needed to walk one sample
   const int64_t units = N * p.nchunk * lane_rows;     // workgroups if each took a single step
   const int64_t target = forced_target > 0 ? forced_target : kTargetBlocks;
+  const int unroll = streams == 1 ? kUnrollFwd : kUnrollBwd;
   int64_t k;
   if (forced_steps > 0) {
     k = forced_steps;
   } else {
-    k = (units + target - 1) / target;
-    if (k < kUnroll) {
-      k = units / 512;
+    // few, tall tiles: about `target` workgroups in all, so that the consumers' merge of tile partials stays short
+    int64_t tiles_wanted = (target + N * p.nchunk - 1) / (N * p.nchunk);
+    if (tiles_wanted < 1) tiles_wanted = 1;
+    k = (lane_rows + tiles_wanted - 1) / tiles_wanted;
+    if (k < unroll) {
+      k = units / kNumCU;  // small problem: keep every CU busy before making tiles taller
       if (k < 1) k = 1;
-      if (k > kUnroll) k = kUnroll;
-    } else {
-      k = (k + kUnroll - 1) / kUnroll * kUnroll;
+      if (k > unroll) k = unroll;
     }
   }
   if (k > lane_rows) k = lane_rows;
   p.tile_rows = (int)(k * p.rpi);
   p.tiles = (int)((R + p.tile_rows - 1) / p.tile_rows);
   p.nblocks = N * p.tiles * p.nchunk;
+  {
+    const int chunk_channels = p.lpr * vec;
+    const int64_t g = (chunk_channels + p.D - 2) / p.D + 1;  // groups a window of chunk_channels can touch
+    p.gmax = (int)(g < G ? g : G);
+  }
   static const int debug = env_int("GNNHWC_DEBUG_PLAN", 0);
   if (debug)
     fprintf(stderr, "[gnnhwc] plan(%s) N=%lld R=%lld C=%lld G=%d D=%d vec=%d cv=%d lpr=%d nchunk=%d rpi=%d tile_rows=%d tiles=%d nblocks=%lld\n",
@@ -244,7 +251,7 @@ int gnnhwc_fwd(const void *x, const void *weight, const void *bias, void *y, voi
   a.eps = eps; a.act = act; a.pdtype = param_dtype; a.sdtype = stats_dtype;
   a.ws = workspace; a.stream = (hipStream_t)stream;
   a.plan = make_plan(N, R, C, G, vector_ok ? vec : 1, 1);
-  if (a.plan.nblocks + 64 > 0x7fffffffLL) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "problem needs too many workgroups");
+  if (a.plan.nchunk > 65535) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "too many channels for this build (C = %lld)", (long long)C);
   hipError_t e;
   switch (dtype) {
     case GN_F32: e = launch_fwd_f32(a); break;
@@ -288,8 +295,7 @@ int gnnhwc_bwd(const void *dy, const void *x, const void *weight, const void *bi
   a.act = act; a.pdtype = param_dtype; a.sdtype = stats_dtype;
   a.ws = workspace; a.stream = (hipStream_t)stream;
   a.plan = make_plan(N, R, C, G, vector_ok ? vec : 1, 2);
-  if (a.plan.nblocks + (C + 255) / 256 + 64 > 0x7fffffffLL)
-    return fail(GNNHWC_ERR_INVALID_ARGUMENT, "problem needs too many workgroups");
+  if (a.plan.nchunk > 65535) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "too many channels for this build (C = %lld)", (long long)C);
   if (N * G > 0x7fffffffLL) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "N * G too large");
   hipError_t e;
   switch (dtype) {
@@ -329,8 +335,8 @@ int gnnhwc_profile_collect(int64_t *launches, double *total_ms) {
 }
 
 const char *gnnhwc_kernel_kind_name(int kind) {
-  static const char *names[GNNHWC_NUM_KERNEL_KINDS] = {"fwd_stats", "fwd_stats_finalize", "fwd_apply", "bwd_reduce",
-                                                       "bwd_finalize", "bwd_dx", "fused_fwd", "fused_bwd"};
+  static const char *names[GNNHWC_NUM_KERNEL_KINDS] = {"fwd_stats", "fwd_stats_compact", "fwd_apply", "bwd_reduce",
+                                                       "bwd_compact", "bwd_dx", "fused_fwd", "fused_bwd"};
   return (kind >= 0 && kind < GNNHWC_NUM_KERNEL_KINDS) ? names[kind] : "";
 }
 

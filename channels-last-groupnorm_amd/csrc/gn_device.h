@@ -45,76 +45,86 @@ __device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
   return __builtin_bit_cast(uint16_t, b);
 }
 
-// ---- lane vectors: VEC elements of T in one (ideally 128-bit) access ----
-template <typename T, int VEC, bool NT> struct LaneVec;
+// ---- lane vectors: VEC elements of T moved by one (ideally 128-bit) access ----
+// raw_t is what travels (and what a lane keeps in registers while more loads are in flight);
+// unpack / pack convert to and from the accumulation type.
+template <typename T, int VEC> struct LaneVec;
 
-template <bool NT> struct LaneVec<float, 4, NT> {
-  static __device__ __forceinline__ void load(const float *p, float (&v)[4]) {
-    f32x4 r = NT ? __builtin_nontemporal_load((const f32x4 *)p) : *(const f32x4 *)p;
-    v[0] = r.x; v[1] = r.y; v[2] = r.z; v[3] = r.w;
-  }
-  static __device__ __forceinline__ void store(float *p, const float (&v)[4]) {
-    f32x4 r = {v[0], v[1], v[2], v[3]};
-    if (NT) __builtin_nontemporal_store(r, (f32x4 *)p); else *(f32x4 *)p = r;
-  }
+template <> struct LaneVec<float, 4> {
+  typedef f32x4 raw_t;
+  static __device__ __forceinline__ raw_t load(const float *p) { return *(const raw_t *)p; }
+  static __device__ __forceinline__ void store(float *p, raw_t r) { *(raw_t *)p = r; }
+  static __device__ __forceinline__ void unpack(raw_t r, float (&v)[4]) { v[0] = r.x; v[1] = r.y; v[2] = r.z; v[3] = r.w; }
+  static __device__ __forceinline__ raw_t pack(const float (&v)[4]) { return raw_t{v[0], v[1], v[2], v[3]}; }
 };
-template <bool NT> struct LaneVec<double, 2, NT> {
-  static __device__ __forceinline__ void load(const double *p, double (&v)[2]) {
-    f64x2 r = NT ? __builtin_nontemporal_load((const f64x2 *)p) : *(const f64x2 *)p;
-    v[0] = r.x; v[1] = r.y;
-  }
-  static __device__ __forceinline__ void store(double *p, const double (&v)[2]) {
-    f64x2 r = {v[0], v[1]};
-    if (NT) __builtin_nontemporal_store(r, (f64x2 *)p); else *(f64x2 *)p = r;
-  }
+template <> struct LaneVec<double, 2> {
+  typedef f64x2 raw_t;
+  static __device__ __forceinline__ raw_t load(const double *p) { return *(const raw_t *)p; }
+  static __device__ __forceinline__ void store(double *p, raw_t r) { *(raw_t *)p = r; }
+  static __device__ __forceinline__ void unpack(raw_t r, double (&v)[2]) { v[0] = r.x; v[1] = r.y; }
+  static __device__ __forceinline__ raw_t pack(const double (&v)[2]) { return raw_t{v[0], v[1]}; }
 };
-template <bool NT> struct LaneVec<f16_t, 8, NT> {
-  static __device__ __forceinline__ void load(const f16_t *p, float (&v)[8]) {
-    f16x8 r = NT ? __builtin_nontemporal_load((const f16x8 *)p) : *(const f16x8 *)p;
+template <> struct LaneVec<f16_t, 8> {
+  typedef f16x8 raw_t;
+  static __device__ __forceinline__ raw_t load(const f16_t *p) { return *(const raw_t *)p; }
+  static __device__ __forceinline__ void store(f16_t *p, raw_t r) { *(raw_t *)p = r; }
+  static __device__ __forceinline__ void unpack(raw_t r, float (&v)[8]) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) v[j] = (float)r[j];
   }
-  static __device__ __forceinline__ void store(f16_t *p, const float (&v)[8]) {
-    f16x8 r;
+  static __device__ __forceinline__ raw_t pack(const float (&v)[8]) {
+    raw_t r;
 #pragma unroll
     for (int j = 0; j < 8; ++j) r[j] = (_Float16)v[j];  // v_cvt_f16_f32, round to nearest even
-    if (NT) __builtin_nontemporal_store(r, (f16x8 *)p); else *(f16x8 *)p = r;
+    return r;
   }
 };
-template <bool NT> struct LaneVec<bf16_t, 8, NT> {
-  static __device__ __forceinline__ void load(const bf16_t *p, float (&v)[8]) {
-    u32x4 r = NT ? __builtin_nontemporal_load((const u32x4 *)p) : *(const u32x4 *)p;
+template <> struct LaneVec<bf16_t, 8> {
+  typedef u32x4 raw_t;
+  static __device__ __forceinline__ raw_t load(const bf16_t *p) { return *(const raw_t *)p; }
+  static __device__ __forceinline__ void store(bf16_t *p, raw_t r) { *(raw_t *)p = r; }
+  static __device__ __forceinline__ void unpack(raw_t r, float (&v)[8]) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       v[2 * j] = bf16_bits_to_float(r[j] << 16);
       v[2 * j + 1] = bf16_bits_to_float(r[j] & 0xffff0000u);
     }
   }
-  static __device__ __forceinline__ void store(bf16_t *p, const float (&v)[8]) {
-    u32x4 r;
+  static __device__ __forceinline__ raw_t pack(const float (&v)[8]) {
+    raw_t r;
 #pragma unroll
     for (int j = 0; j < 4; ++j) r[j] = pack_bf16x2(v[2 * j], v[2 * j + 1]);
-    if (NT) __builtin_nontemporal_store(r, (u32x4 *)p); else *(u32x4 *)p = r;
+    return r;
   }
 };
 // scalar fall-back: any C, any alignment
-template <bool NT> struct LaneVec<float, 1, NT> {
-  static __device__ __forceinline__ void load(const float *p, float (&v)[1]) { v[0] = *p; }
-  static __device__ __forceinline__ void store(float *p, const float (&v)[1]) { *p = v[0]; }
+template <> struct LaneVec<float, 1> {
+  typedef float raw_t;
+  static __device__ __forceinline__ raw_t load(const float *p) { return *p; }
+  static __device__ __forceinline__ void store(float *p, raw_t r) { *p = r; }
+  static __device__ __forceinline__ void unpack(raw_t r, float (&v)[1]) { v[0] = r; }
+  static __device__ __forceinline__ raw_t pack(const float (&v)[1]) { return v[0]; }
 };
-template <bool NT> struct LaneVec<double, 1, NT> {
-  static __device__ __forceinline__ void load(const double *p, double (&v)[1]) { v[0] = *p; }
-  static __device__ __forceinline__ void store(double *p, const double (&v)[1]) { *p = v[0]; }
+template <> struct LaneVec<double, 1> {
+  typedef double raw_t;
+  static __device__ __forceinline__ raw_t load(const double *p) { return *p; }
+  static __device__ __forceinline__ void store(double *p, raw_t r) { *p = r; }
+  static __device__ __forceinline__ void unpack(raw_t r, double (&v)[1]) { v[0] = r; }
+  static __device__ __forceinline__ raw_t pack(const double (&v)[1]) { return v[0]; }
 };
-template <bool NT> struct LaneVec<f16_t, 1, NT> {
-  static __device__ __forceinline__ void load(const f16_t *p, float (&v)[1]) { v[0] = (float)*p; }
-  static __device__ __forceinline__ void store(f16_t *p, const float (&v)[1]) { *p = (_Float16)v[0]; }
+template <> struct LaneVec<f16_t, 1> {
+  typedef f16_t raw_t;
+  static __device__ __forceinline__ raw_t load(const f16_t *p) { return *p; }
+  static __device__ __forceinline__ void store(f16_t *p, raw_t r) { *p = r; }
+  static __device__ __forceinline__ void unpack(raw_t r, float (&v)[1]) { v[0] = (float)r; }
+  static __device__ __forceinline__ raw_t pack(const float (&v)[1]) { return (_Float16)v[0]; }
 };
-template <bool NT> struct LaneVec<bf16_t, 1, NT> {
-  static __device__ __forceinline__ void load(const bf16_t *p, float (&v)[1]) {
-    v[0] = bf16_bits_to_float((uint32_t)p->bits << 16);
-  }
-  static __device__ __forceinline__ void store(bf16_t *p, const float (&v)[1]) { p->bits = float_to_bf16_bits(v[0]); }
+template <> struct LaneVec<bf16_t, 1> {
+  typedef uint16_t raw_t;
+  static __device__ __forceinline__ raw_t load(const bf16_t *p) { return p->bits; }
+  static __device__ __forceinline__ void store(bf16_t *p, raw_t r) { p->bits = r; }
+  static __device__ __forceinline__ void unpack(raw_t r, float (&v)[1]) { v[0] = bf16_bits_to_float((uint32_t)r << 16); }
+  static __device__ __forceinline__ raw_t pack(const float (&v)[1]) { return float_to_bf16_bits(v[0]); }
 };
 
 // ---- runtime-typed scalar access to parameters / statistics (read once per workgroup) ----
@@ -192,69 +202,29 @@ template <int ACT, typename A> __device__ __forceinline__ A act_bwd(A z) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Running statistics: (count, mean, M2) triples merged with Chan's parallel update.  Same
-// quantities as WelfordData / WelfordOps::combine (src/gnnhwc/csrc/Welford.h:8-21,44-65); the
-// variance is the biased one, M2 / n (Welford.h:66-72 with correction 0, gn_kernel.cu:175,254).
+// Statistics are carried as (count, mean, M2) triples, the quantities of WelfordData
+// (src/gnnhwc/csrc/Welford.h:8-21); the variance is the biased one, M2 / n (Welford.h:66-72 with
+// correction 0, gn_kernel.cu:175,254).  Where the reference merges triples pairwise with
+// WelfordOps::combine (Welford.h:44-65), sets of triples are merged here with the equivalent exact
+// two-pass form, which is a pair of plain sums and therefore reduces with fixed butterfly trees:
+//   n = sum n_i,  mean = sum n_i mean_i / n,  M2 = sum (M2_i + n_i (mean_i - mean)^2).
 // ---------------------------------------------------------------------------------------------
 template <typename A> struct Moments {
   A n, mean, m2;
 };
-template <typename A> __device__ __forceinline__ Moments<A> merge(const Moments<A> &a, const Moments<A> &b) {
-  const A n = a.n + b.n;
-  if (b.n == (A)0) return a;
-  const A f = b.n * fast_rcp(n);
-  const A d = b.mean - a.mean;
-  Moments<A> r;
-  r.n = n;
-  r.mean = a.mean + d * f;
-  r.m2 = a.m2 + b.m2 + d * d * a.n * f;
-  return r;
-}
 template <typename A> __device__ __forceinline__ A shfl_xor_acc(A v, int mask, int width) {
   return __shfl_xor(v, mask, width);
 }
-// Butterfly merge over `width` consecutive lanes (power of two <= 64); lane 0 of each segment holds the
-// result of a fixed merge tree, so the outcome does not depend on scheduling.
-template <typename A> __device__ __forceinline__ Moments<A> segment_merge(Moments<A> m, int width) {
-  for (int off = width >> 1; off > 0; off >>= 1) {
-    Moments<A> o;
-    o.n = shfl_xor_acc(m.n, off, width);
-    o.mean = shfl_xor_acc(m.mean, off, width);
-    o.m2 = shfl_xor_acc(m.m2, off, width);
-    // lower lane always merges (self, other), upper lane (other, self): both compute the same value
-    const bool upper = (threadIdx.x & off) != 0;
-    m = upper ? merge(o, m) : merge(m, o);
-  }
-  return m;
-}
+// Butterfly sum over `width` consecutive lanes (power of two <= 64).  Every lane of the segment ends with
+// the same bits: the tree is fixed and floating-point addition is commutative.
 template <typename A> __device__ __forceinline__ A segment_sum(A v, int width) {
-  for (int off = width >> 1; off > 0; off >>= 1) {
-    const A o = shfl_xor_acc(v, off, width);
-    const bool upper = (threadIdx.x & off) != 0;
-    v = upper ? (o + v) : (v + o);
-  }
+  for (int off = width >> 1; off > 0; off >>= 1) v += shfl_xor_acc(v, off, width);
   return v;
 }
-
-// Block index -> (sample, row tile, channel chunk).  Blocks are numbered so that consecutive ids
-// (which the hardware deals round-robin to the 8 XCDs) walk the row tiles of one sample; the
-// second pass of a two-pass operation uses `reversed` so that it starts on the tiles the first
-// pass touched last (still in that XCD's L2) while keeping every tile on the same XCD.
-struct TileCoord {
-  int64_t n;
-  int tile, chunk;
-};
-__device__ __forceinline__ TileCoord decode_block(const Plan &p, int64_t b, bool reversed) {
-  if (reversed) {
-    const int64_t full = p.nblocks & ~(int64_t)7;  // blocks in complete octets; the tail keeps its place
-    if (b < full) b = full - 8 - (b & ~(int64_t)7) + (b & 7);
-  }
-  TileCoord t;
-  t.chunk = (int)(b % p.nchunk);
-  const int64_t nt = b / p.nchunk;
-  t.tile = (int)(nt % p.tiles);
-  t.n = nt / p.tiles;
-  return t;
+__device__ __forceinline__ int pow2_ceil_clamped(int v, int hi) {
+  int p = 1;
+  while (p < v && p < hi) p <<= 1;
+  return p;
 }
 
 }  // namespace gn

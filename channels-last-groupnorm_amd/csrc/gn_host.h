@@ -10,10 +10,10 @@ namespace gn {
 
 enum KernelKind {
   kKindFwdStats = 0,
-  kKindFwdStatsFinalize = 1,
+  kKindFwdStatsCompact = 1,
   kKindFwdApply = 2,
   kKindBwdReduce = 3,
-  kKindBwdFinalize = 4,
+  kKindBwdCompact = 4,
   kKindBwdDx = 5,
   kKindFusedFwd = 6,
   kKindFusedBwd = 7,
@@ -40,27 +40,34 @@ struct BwdArgs {
 
 // Workspace layout, in elements of the accumulation type (float, or double for f64 data).
 struct FwdWorkspace {
-  size_t part, mean, rstd, total;  // element offsets; total = element count
+  size_t part, compact, total;  // element offsets; total = element count
 };
 struct BwdWorkspace {
-  size_t part, sums, coef, total;
+  size_t partC, partG, compactC, compactG, total;
 };
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 inline FwdWorkspace fwd_workspace(const Plan &p) {
   FwdWorkspace w;
   w.part = 0;
-  w.mean = align_up((size_t)p.N * p.tiles * p.nchunk * p.G * 3, 64);
-  w.rstd = w.mean + align_up((size_t)p.N * p.G, 64);
-  w.total = w.rstd + align_up((size_t)p.N * p.G, 64);
+  w.compact = align_up((size_t)p.N * p.tiles * p.nchunk * p.G * 3, 64);  // 3 planes [N][nchunk][G][tiles]
+  w.total = w.compact + align_up((size_t)p.N * p.G * 3, 64);
   return w;
 }
 inline BwdWorkspace bwd_workspace(const Plan &p) {
   BwdWorkspace w;
-  w.part = 0;
-  w.sums = align_up((size_t)p.N * p.tiles * p.C * 2, 64);
-  w.coef = w.sums + align_up((size_t)p.N * p.C * 2, 64);
-  w.total = w.coef + align_up((size_t)p.N * p.G * 2, 64);
+  w.partC = 0;
+  w.partG = align_up((size_t)p.N * p.tiles * p.C * 2, 64);
+  w.compactC = w.partG + align_up((size_t)p.N * p.tiles * p.nchunk * p.G * 2, 64);
+  w.compactG = w.compactC + align_up((size_t)p.N * p.C * 2, 64);
+  w.total = w.compactG + align_up((size_t)p.N * p.G * 2, 64);
   return w;
+}
+// Consumers merge the tile partials of their own groups unless that would be more than
+// kMaxInlineEntries entries per workgroup; then a compaction kernel runs in between.
+inline bool needs_compaction(const Plan &p) {
+  const int chunk_channels = p.lpr * p.vec;
+  const int64_t per_group = (int64_t)p.tiles * ((p.D - 1) / chunk_channels + 2);
+  return per_group * p.gmax > kMaxInlineEntries;
 }
 
 // Bracket one kernel launch with HIP events when profiling is enabled on this thread (gn_api.hip).

@@ -1,123 +1,207 @@
 // The streaming GroupNorm kernels (templates; instantiated once per element type in gn_inst.hip).
 //
-//   forward : stats_kernel -> stats_finalize_kernel -> apply_kernel
-//   backward: bwd_reduce_kernel -> bwd_finalize_kernel -> bwd_dx_kernel
+//   forward : stats_kernel -> [stats_compact_kernel] -> apply_kernel
+//   backward: bwd_reduce_kernel -> [bwd_compact_kernel] -> bwd_dx_kernel
 //
-// Every large kernel walks the same Plan: a workgroup owns a tile of consecutive rows of one sample,
-// each lane owns VEC fixed channels and reads/writes them with one 128-bit access per row, so a
-// wavefront touches whole contiguous rows.  Cross-lane and cross-workgroup reductions use fixed
-// trees and per-tile partial buffers, never floating-point atomics, so results are bit-identical
-// from run to run (the reference has the same property, it contains no atomics either).
+// Every large kernel walks the same Plan: a workgroup owns a tile of consecutive rows of one sample and
+// a chunk of whole 128-byte lines of each row; each lane owns VEC fixed channels and moves them with
+// one 128-bit access per row, two batches of rows in flight at a time.  The producers (stats,
+// bwd_reduce) leave one partial result per tile; the consumers (apply, bwd_dx) merge the partials of
+// the groups they touch in their own prologue, while their first loads are already in flight, so there
+// is no separate finalize launch unless a sample has so many tiles that the merge is first compacted
+// by the bracketed kernels.  All reductions use fixed trees and per-tile buffers, never floating-point
+// atomics: results are bit-identical from run to run (the reference has the same property, it contains
+// no atomics either).
 #pragma once
+#include <type_traits>
+
 #include "gn_device.h"
 
 namespace gn {
 
 template <typename T> using acc_t = typename acc_of<T>::type;
 
-// rows of a tile of `len` rows handled by lane-row ty: ty, ty + rpi, ...
-__device__ __forceinline__ int rows_of(int len, int rpi, int ty) { return len > ty ? (len - ty + rpi - 1) / rpi : 0; }
-
 struct LanePos {
-  TileCoord tc;
+  int64_t n;
+  int tile, chunk;
   int ty, tx, cvi;   // lane row, lane column inside the chunk, lane-vector index inside the row
   int len;           // rows in this tile
   int64_t row0;      // first row of the tile (inside the sample)
+  int cstart, wch;   // first channel and number of channels of this chunk
+  int g_lo, ng;      // first group and number of groups the chunk intersects
+  int rows_base, rows_rem;  // lane row ty owns rows_base + (ty < rows_rem) rows of the tile
+  int rows;          // rows of the tile this lane owns (0 for an idle lane)
   bool active;
 };
-__device__ __forceinline__ LanePos lane_pos(const Plan &p, bool reversed) {
+// `reversed` walks the row tiles from the far end in blocks of eight: the second pass of a two-pass
+// operation then starts on the tiles the first pass touched last, while tile t stays on XCD t mod 8.
+__device__ __forceinline__ LanePos lane_pos(const Plan &p, int64_t n, bool reversed) {
   LanePos l;
-  l.tc = decode_block(p, blockIdx.x, reversed);
+  l.n = n;
+  int t = blockIdx.x;
+  if (reversed) {
+    const int full = p.tiles & ~7;
+    if (t < full) t = full - 8 - (t & ~7) + (t & 7);
+  }
+  l.tile = t;
+  l.chunk = blockIdx.y;
   const int tid = threadIdx.x;
   l.ty = tid / p.lpr;
   l.tx = tid - l.ty * p.lpr;
-  l.cvi = l.tc.chunk * p.lpr + l.tx;
-  l.row0 = (int64_t)l.tc.tile * p.tile_rows;
+  l.cvi = l.chunk * p.lpr + l.tx;
+  l.row0 = (int64_t)l.tile * p.tile_rows;
   const int64_t rem = p.R - l.row0;
   l.len = rem < p.tile_rows ? (int)rem : p.tile_rows;
+  l.rows_base = l.len / p.rpi;
+  l.rows_rem = l.len - l.rows_base * p.rpi;
+  l.cstart = l.chunk * p.lpr * p.vec;
+  const int lanes_here = p.cv - l.chunk * p.lpr < p.lpr ? p.cv - l.chunk * p.lpr : p.lpr;
+  l.wch = lanes_here * p.vec;
+  l.g_lo = l.cstart / p.D;
+  l.ng = (l.cstart + l.wch - 1) / p.D - l.g_lo + 1;
   l.active = l.ty < p.rpi && l.cvi < p.cv;
+  l.rows = l.active ? l.rows_base + (l.ty < l.rows_rem ? 1 : 0) : 0;
   return l;
 }
 
-// a = rstd * gamma, b = beta - mean * a: normalise + affine as one FMA per element
-// (same folding as src/gnnhwc/csrc/gn_kernel.cu:350-379, 601-602, 783-784).
-template <typename A, int VEC>
-__device__ __forceinline__ void affine_coeffs(const Plan &p, const LanePos &l, const void *mean, const void *rstd,
-                                              int sdtype, const void *w, const void *b, int pdtype, A (&sa)[VEC],
-                                              A (&sb)[VEC]) {
-#pragma unroll
-  for (int j = 0; j < VEC; ++j) {
-    const int c = l.cvi * VEC + j;
-    const int g = c / p.D;
-    const int64_t ng = l.tc.n * p.G + g;
-    const A mu = load_scalar<A>(mean, ng, sdtype);
-    const A rs = load_scalar<A>(rstd, ng, sdtype);
-    const A gamma = w ? load_scalar<A>(w, c, pdtype) : (A)1;
-    const A beta = b ? load_scalar<A>(b, c, pdtype) : (A)0;
-    sa[j] = rs * gamma;
-    sb[j] = beta - mu * sa[j];
+// A lane walks its rows in batches of U and keeps two batches of raw vectors in registers: while batch b
+// is being consumed the loads of batch b + 1 are already in flight.  issue(sel, b) starts the loads of
+// batch b into buffer `sel` (std::integral_constant 0 / 1); consume(sel, b) uses them.  The caller issues
+// batch 0 itself, before any prologue it wants to hide behind those loads.
+// Row u of batch b is the lane's row min(b U + u, rows - 1): the trailing batch re-reads the last row
+// instead of branching, consumers that accumulate weight such duplicates with 0, consumers that store
+// simply store the same values again.
+template <typename ISSUE, typename CONSUME>
+__device__ __forceinline__ void double_buffered(int nb, ISSUE &&issue, CONSUME &&consume) {
+  using B0 = std::integral_constant<int, 0>;
+  using B1 = std::integral_constant<int, 1>;
+  for (int b = 0; b < nb; b += 2) {
+    if (b + 1 < nb) issue(B1{}, b + 1);
+    consume(B0{}, b);
+    if (b + 1 < nb) {
+      if (b + 2 < nb) issue(B0{}, b + 2);
+      consume(B1{}, b + 1);
+    }
   }
+}
+__device__ __forceinline__ int clamp_row(int idx, int rows) { return idx < rows ? idx : rows - 1; }
+
+template <typename PT, typename A> __device__ __forceinline__ A load_param(const void *p, int64_t i) {
+  A v[1];
+  LaneVec<PT, 1>::unpack(LaneVec<PT, 1>::load((const PT *)p + i), v);
+  return v[0];
+}
+template <typename PT, typename A> __device__ __forceinline__ void store_param(void *p, int64_t i, A x) {
+  const A v[1] = {x};
+  LaneVec<PT, 1>::store((PT *)p + i, LaneVec<PT, 1>::pack(v));
+}
+
+// Per-group tile partials are stored as planes of one field each, laid out [N][nchunk][G][tiles]: the
+// entries a consumer merges for one group (all tiles of the one or two chunks that hold the group) are
+// contiguous, so the merge reads them with coalesced loads.
+__device__ __forceinline__ int64_t group_slot(const PartialGeo &q, int G, int64_t n, int t, int k, int g) {
+  return ((n * q.nchunk + k) * G + g) * q.tiles + t;
+}
+__device__ __forceinline__ int64_t group_plane(const PartialGeo &q, int G, int64_t N) {
+  return N * q.nchunk * G * q.tiles;
+}
+// Chunks [k_lo, k_lo + nk) of the producer hold pieces of group g.
+__device__ __forceinline__ void group_chunks(const PartialGeo &q, int D, int g, int &k_lo, int &nk) {
+  k_lo = (g * D) / q.chunk_channels;
+  nk = ((g + 1) * D - 1) / q.chunk_channels - k_lo + 1;
+}
+// Lanes per group for a consumer's merge of tile partials.
+__device__ __forceinline__ int merge_lanes(const PartialGeo &q, int D) {
+  return pow2_ceil_clamped(q.tiles * ((D - 1) / q.chunk_channels + 2), 64);
+}
+// Channels [ca, cb) (relative to the chunk) of group g that lie inside the chunk.
+__device__ __forceinline__ void group_span(const Plan &p, const LanePos &l, int g, int &ca, int &cb) {
+  ca = (g * p.D > l.cstart ? g * p.D : l.cstart) - l.cstart;
+  cb = ((g + 1) * p.D < l.cstart + l.wch ? (g + 1) * p.D : l.cstart + l.wch) - l.cstart;
 }
 
 // ---------------------------------------------------------------------------------------------
-// Forward pass 1: per-tile (count, mean, M2) of every group the tile touches.
-// Does the work of compute_stats_pt1 (src/gnnhwc/csrc/gn_kernel.cu:132-224).  Each lane folds
-// kUnroll rows at a time with an exact two-pass mean / sum-of-squares on the values it holds in
-// registers and merges that block into its running moments (one reciprocal per kUnroll rows instead
-// of the per-element division of WelfordOps::reduce, Welford.h:30-42).
-//   part : [N][tiles][nchunk][G][3] accumulation type; only the groups a chunk intersects are written.
+// Running per-channel statistics of one lane over its rows of the tile.  Each batch of rows is folded
+// with an exact two-pass mean / sum of squares on the values held in registers and merged into the
+// running moments with Chan's update: one reciprocal per batch instead of the per-element division of
+// WelfordOps::reduce (src/gnnhwc/csrc/Welford.h:30-42).
 // ---------------------------------------------------------------------------------------------
-template <typename T, int VEC>
-__global__ __launch_bounds__(kBlock) void stats_kernel(const T *__restrict__ x, acc_t<T> *__restrict__ part, Plan p) {
+template <typename T, int VEC, int U>
+__device__ __forceinline__ void fold_batch(const typename LaneVec<T, VEC>::raw_t (&raw)[U], int m, acc_t<T> &cnt,
+                                           acc_t<T> (&mean)[VEC], acc_t<T> (&m2)[VEC]) {
   using A = acc_t<T>;
-  __shared__ A sm_mean[kBlock * VEC];
-  __shared__ A sm_m2[kBlock * VEC];
-  const LanePos l = lane_pos(p, false);
-  const int W = p.lpr * VEC;
+  A s[VEC], qq[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) { s[j] = (A)0; qq[j] = (A)0; }
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const A keep = u < m ? (A)1 : (A)0;
+    A v[VEC];
+    LaneVec<T, VEC>::unpack(raw[u], v);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) s[j] += keep * v[j];
+  }
+  const A mf = (A)m;
+  const A inv_m = fast_rcp(mf);
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) s[j] *= inv_m;  // batch mean
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const A keep = u < m ? (A)1 : (A)0;
+    A v[VEC];
+    LaneVec<T, VEC>::unpack(raw[u], v);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) { const A d = v[j] - s[j]; qq[j] += keep * d * d; }
+  }
+  const A nn = cnt + mf;
+  const A f = mf * fast_rcp(nn);
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    const A d = s[j] - mean[j];
+    mean[j] += d * f;
+    m2[j] += qq[j] + d * d * cnt * f;
+  }
+  cnt = nn;
+}
 
+template <typename T, int VEC, int U>
+__device__ __forceinline__ void lane_stats(const T *__restrict__ x, const Plan &p, const LanePos &l,
+                                           acc_t<T> (&mean)[VEC], acc_t<T> (&m2)[VEC]) {
+  using A = acc_t<T>;
+  using LV = LaneVec<T, VEC>;
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) { mean[j] = (A)0; m2[j] = (A)0; }
+  A cnt = (A)0;
+  const int rows = l.rows;
+  const int nb = (rows + U - 1) / U;
+  const T *base = x + ((l.n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC);
+  const int64_t step = (int64_t)p.rpi * p.C;
+  typename LV::raw_t buf0[U], buf1[U];
+  auto issue = [&](auto sel, int b) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const T *src = base + (int64_t)clamp_row(b * U + u, rows) * step;
+      if constexpr (decltype(sel)::value == 0) buf0[u] = LV::load(src);
+      else buf1[u] = LV::load(src);
+    }
+  };
+  auto consume = [&](auto sel, int b) {
+    const int m = rows - b * U < U ? rows - b * U : U;
+    if constexpr (decltype(sel)::value == 0) fold_batch<T, VEC, U>(buf0, m, cnt, mean, m2);
+    else fold_batch<T, VEC, U>(buf1, m, cnt, mean, m2);
+  };
+  if (nb > 0) issue(std::integral_constant<int, 0>{}, 0);
+  double_buffered(nb, issue, consume);
+}
+
+// Merge the per-lane moments of a workgroup into one (count, mean, M2) triple per group of the chunk and
+// hand each to emit(g, count, mean, M2) (called by one lane per group).  Uses the exact two-pass form,
+// first across the lane rows of a channel, then across the channels of a group.
+template <typename A, int VEC, typename EMIT>
+__device__ __forceinline__ void block_group_moments(const Plan &p, const LanePos &l, const A (&mean)[VEC],
+                                                    const A (&m2)[VEC], A *sm_mean, A *sm_m2, EMIT &&emit) {
+  const int W = p.lpr * VEC;
   if (l.active) {
-    A mean[VEC], m2[VEC];
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) { mean[j] = (A)0; m2[j] = (A)0; }
-    A cnt = (A)0;
-    const T *px = x + ((l.tc.n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC);
-    const int64_t step = (int64_t)p.rpi * p.C;
-    int lr = l.ty;
-    for (; lr + (kUnroll - 1) * p.rpi < l.len; lr += kUnroll * p.rpi) {
-      A v[kUnroll][VEC];
-#pragma unroll
-      for (int u = 0; u < kUnroll; ++u) LaneVec<T, VEC, false>::load(px + u * step, v[u]);
-      px += kUnroll * step;
-      const A n = cnt + (A)kUnroll;
-      const A f = (A)kUnroll * fast_rcp(n);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        A s = v[0][j];
-#pragma unroll
-        for (int u = 1; u < kUnroll; ++u) s += v[u][j];
-        const A mb = s * ((A)1 / (A)kUnroll);
-        A q = (A)0;
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) { const A d = v[u][j] - mb; q += d * d; }
-        const A d = mb - mean[j];
-        mean[j] += d * f;
-        m2[j] += q + d * d * cnt * f;
-      }
-      cnt = n;
-    }
-    for (; lr < l.len; lr += p.rpi) {
-      A v[VEC];
-      LaneVec<T, VEC, false>::load(px, v);
-      px += step;
-      cnt += (A)1;
-      const A inv = fast_rcp(cnt);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        const A d = v[j] - mean[j];
-        mean[j] += d * inv;
-        m2[j] += d * (v[j] - mean[j]);
-      }
-    }
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
       sm_mean[l.ty * W + l.tx * VEC + j] = mean[j];
@@ -125,345 +209,554 @@ __global__ __launch_bounds__(kBlock) void stats_kernel(const T *__restrict__ x, 
     }
   }
   __syncthreads();
-
-  // merge the per-(lane row, channel) moments of each group this chunk intersects: 16 lanes per group
-  const int cstart = l.tc.chunk * p.lpr * VEC;
-  const int lanes_here = p.cv - l.tc.chunk * p.lpr < p.lpr ? p.cv - l.tc.chunk * p.lpr : p.lpr;
-  const int cend = cstart + lanes_here * VEC;
-  const int g_lo = cstart / p.D, g_hi = (cend - 1) / p.D;
-  const int ng = g_hi - g_lo + 1;
-  constexpr int L = 16;
-  constexpr int NSUB = kBlock / L;
-  const int sub = threadIdx.x / L, sl = threadIdx.x % L;
-  for (int base = 0; base < ng; base += NSUB) {
-    const int gi = base + sub;
-    const int g = g_lo + gi;
-    Moments<A> m = {(A)0, (A)0, (A)0};
-    if (gi < ng) {
-      const int ca = (g * p.D > cstart ? g * p.D : cstart) - cstart;
-      const int cb = ((g + 1) * p.D < cend ? (g + 1) * p.D : cend) - cstart;
-      for (int ety = 0; ety < p.rpi; ++ety) {
-        const int rc = rows_of(l.len, p.rpi, ety);
-        if (rc == 0) break;
-        for (int c = ca + sl; c < cb; c += L) {
-          const Moments<A> e = {(A)rc, sm_mean[ety * W + c], sm_m2[ety * W + c]};
-          m = merge(m, e);
-        }
-      }
+  const int rows_used = l.len < p.rpi ? l.len : p.rpi;
+  for (int c = threadIdx.x; c < l.wch; c += kBlock) {
+    A sm = (A)0;
+    for (int ty = 0; ty < rows_used; ++ty) sm += (A)(l.rows_base + (ty < l.rows_rem ? 1 : 0)) * sm_mean[ty * W + c];
+    const A mu = sm / (A)l.len;
+    A s2 = (A)0;
+    for (int ty = 0; ty < rows_used; ++ty) {
+      const A d = sm_mean[ty * W + c] - mu;
+      s2 += sm_m2[ty * W + c] + (A)(l.rows_base + (ty < l.rows_rem ? 1 : 0)) * d * d;
     }
-    m = segment_merge(m, L);
-    if (gi < ng && sl == 0) {
-      const int64_t slot = ((l.tc.n * p.tiles + l.tc.tile) * p.nchunk + l.tc.chunk) * p.G + g;
-      part[slot * 3 + 0] = m.n;
-      part[slot * 3 + 1] = m.mean;
-      part[slot * 3 + 2] = m.m2;
-    }
+    sm_mean[c] = mu;  // the column's result replaces its row 0 (only this thread touches the column)
+    sm_m2[c] = s2;
   }
+  __syncthreads();
+  const int L = pow2_ceil_clamped(p.D < l.wch ? p.D : l.wch, 64);
+  const int nseg = kBlock / L;
+  const int seg = threadIdx.x / L, sl = threadIdx.x % L;
+  for (int base = 0; base < l.ng; base += nseg) {
+    const int gi = base + seg;
+    const int g = l.g_lo + gi;
+    const bool valid = gi < l.ng;
+    int ca = 0, cb = 0;
+    if (valid) group_span(p, l, g, ca, cb);
+    A sm = (A)0;
+    for (int c = ca + sl; c < cb; c += L) sm += sm_mean[c];
+    sm = segment_sum(sm, L);
+    const A nch = (A)(cb - ca);
+    const A mu = valid ? sm / nch : (A)0;
+    A s2 = (A)0;
+    for (int c = ca + sl; c < cb; c += L) {
+      const A d = sm_mean[c] - mu;
+      s2 += sm_m2[c] + (A)l.len * d * d;
+    }
+    s2 = segment_sum(s2, L);
+    if (valid && sl == 0) emit(g, nch * (A)l.len, mu, s2);
+  }
+  __syncthreads();  // the LDS arrays may be reused by the caller
 }
 
 // ---------------------------------------------------------------------------------------------
-// Forward pass 2: merge the tile partials of one (n, g) per wavefront, in slot order, and produce
-// mean and rstd = 1 / sqrt(M2 / n + eps).  Does the work of compute_stats_pt2
-// (src/gnnhwc/csrc/gn_kernel.cu:226-292), except that the accumulation-type copies kept in the
-// workspace (ws_mean / ws_rstd) feed the apply kernel, so rounding mean / rstd to a 16-bit output
-// type (gn_kernel.cu:290-291) does not touch y.
+// Forward pass 1: per-tile (count, mean, M2) of every group the tile touches.
+// Does the work of compute_stats_pt1 (src/gnnhwc/csrc/gn_kernel.cu:132-224).
+//   part : 3 planes [N][nchunk][G][tiles]; only the groups a chunk intersects are written.
+// ---------------------------------------------------------------------------------------------
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) void stats_kernel(
+    const T *__restrict__ x, acc_t<T> *__restrict__ part, Plan p) {
+  using A = acc_t<T>;
+  __shared__ A sm_mean[kBlock * VEC];
+  __shared__ A sm_m2[kBlock * VEC];
+  const PartialGeo q = {p.tiles, p.nchunk, p.lpr * p.vec};
+  const int64_t plane = group_plane(q, p.G, p.N);
+  for (int64_t n = blockIdx.z; n < p.N; n += gridDim.z) {
+    const LanePos l = lane_pos(p, n, false);
+    A mean[VEC], m2[VEC];
+    lane_stats<T, VEC, kUnrollFwd>(x, p, l, mean, m2);
+    block_group_moments<A, VEC>(p, l, mean, m2, sm_mean, sm_m2, [&](int g, A cnt, A mu, A s2) {
+      const int64_t slot = group_slot(q, p.G, n, l.tile, l.chunk, g);
+      part[slot] = cnt;
+      part[plane + slot] = mu;
+      part[2 * plane + slot] = s2;
+    });
+  }
+}
+
+// Merge the P = tiles * (chunks holding a piece of g) partial triples of group g with `L` lanes; every
+// lane of the segment returns the merged triple (exact two-pass form).
+template <typename A>
+__device__ __forceinline__ Moments<A> merge_group_partials(const A *__restrict__ part, int64_t plane, const PartialGeo &q,
+                                                           int G, int D, int64_t n, int g, bool valid, int L, int sl) {
+  int k_lo = 0, nk = 1;
+  if (valid) group_chunks(q, D, g, k_lo, nk);
+  const int P = valid ? q.tiles * nk : 0;
+  // entries of chunk k_lo .. k_lo + nk - 1 are contiguous runs of q.tiles values each
+  const int64_t base = group_slot(q, G, n, 0, k_lo, g);
+  const int64_t kstride = (int64_t)G * q.tiles;
+  A sn = (A)0, sm = (A)0;
+  for (int e = sl; e < P; e += L) {
+    const int k = e / q.tiles, t = e - k * q.tiles;
+    const int64_t slot = base + k * kstride + t;
+    const A cn = part[slot];
+    sn += cn;
+    sm += cn * part[plane + slot];
+  }
+  sn = segment_sum(sn, L);
+  sm = segment_sum(sm, L);
+  Moments<A> r;
+  r.n = sn;
+  r.mean = valid ? sm / sn : (A)0;
+  A s2 = (A)0;
+  for (int e = sl; e < P; e += L) {
+    const int k = e / q.tiles, t = e - k * q.tiles;
+    const int64_t slot = base + k * kstride + t;
+    const A d = part[plane + slot] - r.mean;
+    s2 += part[2 * plane + slot] + part[slot] * d * d;
+  }
+  r.m2 = segment_sum(s2, L);
+  return r;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Optional forward pass 1b (only when a sample has too many tiles for the consumers to merge
+// themselves): one wavefront per (n, g) merges the tile partials into a single triple.
+//   out : 3 planes [N][G]
 // ---------------------------------------------------------------------------------------------
 template <typename A>
-__global__ __launch_bounds__(kBlock) void stats_finalize_kernel(const A *__restrict__ part, A *__restrict__ ws_mean,
-                                                                A *__restrict__ ws_rstd, void *mean_out, void *rstd_out,
-                                                                int sdtype, A eps, Plan p) {
+__global__ __launch_bounds__(kBlock) void stats_compact_kernel(const A *__restrict__ part, A *__restrict__ out,
+                                                               PartialGeo q, Plan p) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int64_t item = (int64_t)blockIdx.x * (kBlock / 64) + wave;
   const bool valid = item < p.N * p.G;
-  Moments<A> m = {(A)0, (A)0, (A)0};
-  if (valid) {
-    const int64_t n = item / p.G;
-    const int g = (int)(item - n * p.G);
-    const int chunk_w = p.lpr * p.vec;
-    const int k_lo = (g * p.D) / chunk_w, k_hi = ((g + 1) * p.D - 1) / chunk_w;
-    const int nk = k_hi - k_lo + 1;
-    const int entries = p.tiles * nk;
-    for (int e = lane; e < entries; e += 64) {
-      const int t = e / nk, k = k_lo + (e - t * nk);
-      const int64_t slot = ((n * p.tiles + t) * p.nchunk + k) * p.G + g;
-      const Moments<A> q = {part[slot * 3 + 0], part[slot * 3 + 1], part[slot * 3 + 2]};
-      m = merge(m, q);
-    }
-  }
-  m = segment_merge(m, 64);
+  const int64_t n = valid ? item / p.G : 0;
+  const int g = valid ? (int)(item - n * p.G) : 0;
+  const Moments<A> m = merge_group_partials<A>(part, group_plane(q, p.G, p.N), q, p.G, p.D, n, g, valid, 64, lane);
   if (valid && lane == 0) {
-    const A var = m.m2 / m.n;
-    const A rs = (A)1 / sqrt(var + eps);
-    ws_mean[item] = m.mean;
-    ws_rstd[item] = rs;
-    store_scalar<A>(mean_out, item, sdtype, m.mean);
-    store_scalar<A>(rstd_out, item, sdtype, rs);
+    const int64_t oplane = p.N * p.G;
+    out[item] = m.n;
+    out[oplane + item] = m.mean;
+    out[2 * oplane + item] = m.m2;
   }
 }
 
-// ---------------------------------------------------------------------------------------------
-// Forward pass 3: y = act(x * a + b).  Does the work of scale_shift_kernel
-// (src/gnnhwc/csrc/gn_kernel.cu:305-412) for every shape with one code path (no R % 8 fast / slow split).
-// ---------------------------------------------------------------------------------------------
-template <typename T, int VEC, int ACT>
-__global__ __launch_bounds__(kBlock) void apply_kernel(const T *__restrict__ x, T *__restrict__ y,
-                                                       const acc_t<T> *__restrict__ ws_mean,
-                                                       const acc_t<T> *__restrict__ ws_rstd, const void *w, const void *b,
-                                                       int pdtype, Plan p) {
-  using A = acc_t<T>;
-  const LanePos l = lane_pos(p, true);
-  if (!l.active) return;
-  constexpr int acc_dtype = sizeof(A) == 8 ? GN_F64 : GN_F32;
-  A sa[VEC], sb[VEC];
-  affine_coeffs<A, VEC>(p, l, ws_mean, ws_rstd, acc_dtype, w, b, pdtype, sa, sb);
-  const int64_t off = (l.tc.n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC;
-  const T *px = x + off;
-  T *py = y + off;
-  const int64_t step = (int64_t)p.rpi * p.C;
-  int lr = l.ty;
-  for (; lr + (kUnroll - 1) * p.rpi < l.len; lr += kUnroll * p.rpi) {
-    A v[kUnroll][VEC];
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) LaneVec<T, VEC, true>::load(px + u * step, v[u]);
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) v[u][j] = act_fwd<ACT, A>(v[u][j] * sa[j] + sb[j]);
-      LaneVec<T, VEC, true>::store(py + u * step, v[u]);
+// Consumer prologue of the forward: merge the tile partials of the chunk's groups into mean / rstd
+// (compute_stats_pt2, src/gnnhwc/csrc/gn_kernel.cu:226-292: rstd = 1 / sqrt(M2 / n + eps)), leave them in
+// LDS indexed by (g - g_lo), and let the workgroups of row tile 0 report them to the caller's outputs.
+template <typename A>
+__device__ __forceinline__ void merge_chunk_stats(const A *__restrict__ part, const PartialGeo &q, const Plan &p,
+                                                  const LanePos &l, A eps, A *sm_mu, A *sm_rs, void *mean_out,
+                                                  void *rstd_out, int sdtype) {
+  const int L = merge_lanes(q, p.D);
+  const int nseg = kBlock / L;
+  const int seg = threadIdx.x / L, sl = threadIdx.x % L;
+  const int64_t plane = group_plane(q, p.G, p.N);
+  for (int base = 0; base < l.ng; base += nseg) {
+    const int gi = base + seg;
+    const bool valid = gi < l.ng;
+    const int g = l.g_lo + gi;
+    const Moments<A> m = merge_group_partials<A>(part, plane, q, p.G, p.D, l.n, g, valid, L, sl);
+    if (valid && sl == 0) {
+      const A rs = (A)1 / sqrt(m.m2 / m.n + eps);
+      sm_mu[gi] = m.mean;
+      sm_rs[gi] = rs;
+      if (l.tile == 0 && g * p.D >= l.cstart) {  // the chunk where the group starts reports it
+        store_scalar<A>(mean_out, l.n * p.G + g, sdtype, m.mean);
+        store_scalar<A>(rstd_out, l.n * p.G + g, sdtype, rs);
+      }
     }
-    px += kUnroll * step;
-    py += kUnroll * step;
   }
-  for (; lr < l.len; lr += p.rpi) {
-    A v[VEC];
-    LaneVec<T, VEC, true>::load(px, v);
+  __syncthreads();
+}
+// Backward: the caller's mean / rstd of the chunk's groups, staged in LDS the same way.
+template <typename A>
+__device__ __forceinline__ void stage_chunk_stats(const void *mean, const void *rstd, int sdtype, const Plan &p,
+                                                  const LanePos &l, A *sm_mu, A *sm_rs) {
+  for (int gi = threadIdx.x; gi < l.ng; gi += kBlock) {
+    sm_mu[gi] = load_scalar<A>(mean, l.n * p.G + l.g_lo + gi, sdtype);
+    sm_rs[gi] = load_scalar<A>(rstd, l.n * p.G + l.g_lo + gi, sdtype);
+  }
+}
+
+// a = rstd * gamma, b = beta - mean * a: normalise + affine as one FMA per element (same folding as
+// src/gnnhwc/csrc/gn_kernel.cu:350-379, 601-602, 783-784).  Group statistics come from LDS; optional
+// per-group extras (the backward's coef1 / coef2) are fetched alongside.
+template <typename A, typename PT, int VEC, bool EXTRA>
+__device__ __forceinline__ void lane_coeffs(const Plan &p, const LanePos &l, const void *w, const void *b,
+                                            const A *sm_mu, const A *sm_rs, const A *sm_c1, const A *sm_c2, A (&sa)[VEC],
+                                            A (&sb)[VEC], A (&c1)[VEC], A (&c2)[VEC]) {
+  const int c = l.cvi * VEC;
+  A gamma[VEC], beta[VEC];
+  if (w) {
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) v[j] = act_fwd<ACT, A>(v[j] * sa[j] + sb[j]);
-    LaneVec<T, VEC, true>::store(py, v);
-    px += step;
-    py += step;
+    for (int j = 0; j < VEC; ++j) gamma[j] = load_param<PT, A>(w, c + j);
+  } else {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) gamma[j] = (A)1;
+  }
+  if (b) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) beta[j] = load_param<PT, A>(b, c + j);
+  } else {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) beta[j] = (A)0;
+  }
+  int gi = c / p.D;
+  int rem = c - gi * p.D;
+  gi -= l.g_lo;
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    sa[j] = sm_rs[gi] * gamma[j];
+    sb[j] = beta[j] - sm_mu[gi] * sa[j];
+    if (EXTRA) {
+      c1[j] = sm_c1[gi];
+      c2[j] = sm_c2[gi];
+    }
+    ++rem;
+    const bool wrap = rem == p.D;
+    rem = wrap ? 0 : rem;
+    gi += wrap ? 1 : 0;
   }
 }
 
 // ---------------------------------------------------------------------------------------------
-// Backward pass 1: per-tile, per-channel S1 = sum g * x and S2 = sum g with g = dy * act'(x a + b)
-// recomputed from x.  Does the work of width_reduce (src/gnnhwc/csrc/gn_kernel.cu:557-646).
-//   part : [N][tiles][C][2] accumulation type.
+// Forward pass 2: y = act(x * a + b) (scale_shift_kernel, src/gnnhwc/csrc/gn_kernel.cu:305-412), for every
+// shape with one code path (no R % 8 fast / slow split).  y is computed from the unrounded mean / rstd
+// whatever type the reported statistics have (cf. gn_kernel.cu:290-291).
 // ---------------------------------------------------------------------------------------------
-template <typename T, int VEC, int ACT>
-__global__ __launch_bounds__(kBlock) void bwd_reduce_kernel(const T *__restrict__ x, const T *__restrict__ dy,
-                                                            const void *mean, const void *rstd, int sdtype, const void *w,
-                                                            const void *b, int pdtype, acc_t<T> *__restrict__ part,
-                                                            Plan p) {
+template <typename T, typename PT, int VEC, int ACT>
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) void apply_kernel(
+    const T *__restrict__ x, T *__restrict__ y, const acc_t<T> *__restrict__ part, PartialGeo q, const void *w,
+    const void *b, void *mean_out, void *rstd_out, int sdtype, acc_t<T> eps, Plan p) {
   using A = acc_t<T>;
+  using LV = LaneVec<T, VEC>;
+  constexpr int U = kUnrollFwd;
+  __shared__ A sm_mu[kBlock * VEC];
+  __shared__ A sm_rs[kBlock * VEC];
+  for (int64_t n = blockIdx.z; n < p.N; n += gridDim.z) {
+    const LanePos l = lane_pos(p, n, true);
+    const int rows = l.rows;
+    const int nb = (rows + U - 1) / U;
+    const int64_t off = (n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC;
+    const int64_t step = (int64_t)p.rpi * p.C;
+    typename LV::raw_t buf0[U], buf1[U];
+    A sa[VEC], sb[VEC], unused1[VEC], unused2[VEC];
+    auto issue = [&](auto sel, int bi) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const T *src = x + off + (int64_t)clamp_row(bi * U + u, rows) * step;
+        if constexpr (decltype(sel)::value == 0) buf0[u] = LV::load(src);
+        else buf1[u] = LV::load(src);
+      }
+    };
+    auto consume = [&](auto sel, int bi) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        A v[VEC];
+        if constexpr (decltype(sel)::value == 0) LV::unpack(buf0[u], v);
+        else LV::unpack(buf1[u], v);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] = act_fwd<ACT, A>(v[j] * sa[j] + sb[j]);
+        LV::store(y + off + (int64_t)clamp_row(bi * U + u, rows) * step, LV::pack(v));
+      }
+    };
+    if (nb > 0) issue(std::integral_constant<int, 0>{}, 0);  // in flight while the statistics are merged
+    merge_chunk_stats<A>(part, q, p, l, eps, sm_mu, sm_rs, mean_out, rstd_out, sdtype);
+    if (nb > 0) {
+      lane_coeffs<A, PT, VEC, false>(p, l, w, b, sm_mu, sm_rs, nullptr, nullptr, sa, sb, unused1, unused2);
+      double_buffered(nb, issue, consume);
+    }
+    __syncthreads();  // sm_mu / sm_rs are rewritten for the next sample of a wrapped grid
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Backward pass 1: per tile, per channel S1 = sum g x and S2 = sum g with g = dy * act'(x a + b)
+// recomputed from x (width_reduce, src/gnnhwc/csrc/gn_kernel.cu:557-646), and per tile, per group
+// A = sum_c gamma_c S1_c and B = sum_c gamma_c S2_c (the group sums of compute_bwd_scale_biases,
+// gn_kernel.cu:786-797).
+//   partC : [N][tiles][C][2]      partG : 2 planes [N][nchunk][G][tiles]
+// ---------------------------------------------------------------------------------------------
+template <typename T, typename PT, int VEC, int ACT>
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) void bwd_reduce_kernel(
+    const T *__restrict__ x, const T *__restrict__ dy, const void *mean, const void *rstd, int sdtype, const void *w,
+    const void *b, acc_t<T> *__restrict__ partC, acc_t<T> *__restrict__ partG, Plan p) {
+  using A = acc_t<T>;
+  using LV = LaneVec<T, VEC>;
+  constexpr int U = kUnrollBwd;
   __shared__ A sm1[kBlock * VEC];
   __shared__ A sm2[kBlock * VEC];
-  const LanePos l = lane_pos(p, false);
-  const int W = p.lpr * VEC;
-  if (l.active) {
-    A sa[VEC], sb[VEC], s1[VEC], s2[VEC];
-    affine_coeffs<A, VEC>(p, l, mean, rstd, sdtype, w, b, pdtype, sa, sb);
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) { s1[j] = (A)0; s2[j] = (A)0; }
-    const int64_t off = (l.tc.n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC;
-    const T *px = x + off;
-    const T *pdy = dy + off;
+  __shared__ A sm_mu[kBlock * VEC];
+  __shared__ A sm_rs[kBlock * VEC];
+  const PartialGeo q = {p.tiles, p.nchunk, p.lpr * p.vec};
+  const int64_t plane = group_plane(q, p.G, p.N);
+  for (int64_t n = blockIdx.z; n < p.N; n += gridDim.z) {
+    const LanePos l = lane_pos(p, n, false);
+    const int W = p.lpr * VEC;
+    const int rows = l.rows;
+    const int nb = (rows + U - 1) / U;
+    const int64_t off = (n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC;
     const int64_t step = (int64_t)p.rpi * p.C;
-    int lr = l.ty;
-    for (; lr + (kUnroll - 1) * p.rpi < l.len; lr += kUnroll * p.rpi) {
-      A vx[kUnroll][VEC], vd[kUnroll][VEC];
+    typename LV::raw_t bx0[U], bx1[U], bd0[U], bd1[U];
+    A sa[VEC], sb[VEC], s1[VEC], s2[VEC], unused1[VEC], unused2[VEC];
+    auto issue = [&](auto sel, int bi) {
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) {
-        LaneVec<T, VEC, false>::load(px + u * step, vx[u]);
-        LaneVec<T, VEC, false>::load(pdy + u * step, vd[u]);
+      for (int u = 0; u < U; ++u) {
+        const int64_t o = off + (int64_t)clamp_row(bi * U + u, rows) * step;
+        if constexpr (decltype(sel)::value == 0) { bx0[u] = LV::load(x + o); bd0[u] = LV::load(dy + o); }
+        else { bx1[u] = LV::load(x + o); bd1[u] = LV::load(dy + o); }
       }
-      px += kUnroll * step;
-      pdy += kUnroll * step;
+    };
+    auto consume = [&](auto sel, int bi) {
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) {
+      for (int u = 0; u < U; ++u) {
+        const A keep = bi * U + u < rows ? (A)1 : (A)0;
+        A vx[VEC], vd[VEC];
+        if constexpr (decltype(sel)::value == 0) { LV::unpack(bx0[u], vx); LV::unpack(bd0[u], vd); }
+        else { LV::unpack(bx1[u], vx); LV::unpack(bd1[u], vd); }
 #pragma unroll
         for (int j = 0; j < VEC; ++j) {
-          const A g = vd[u][j] * act_bwd<ACT, A>(vx[u][j] * sa[j] + sb[j]);
-          s1[j] += g * vx[u][j];
+          const A g = keep * vd[j] * act_bwd<ACT, A>(vx[j] * sa[j] + sb[j]);
+          s1[j] += g * vx[j];
           s2[j] += g;
         }
       }
-    }
-    for (; lr < l.len; lr += p.rpi) {
-      A vx[VEC], vd[VEC];
-      LaneVec<T, VEC, false>::load(px, vx);
-      LaneVec<T, VEC, false>::load(pdy, vd);
-      px += step;
-      pdy += step;
+    };
+    if (nb > 0) issue(std::integral_constant<int, 0>{}, 0);
+    stage_chunk_stats<A>(mean, rstd, sdtype, p, l, sm_mu, sm_rs);
+    __syncthreads();
+    if (l.active) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) { s1[j] = (A)0; s2[j] = (A)0; }
+      if (nb > 0) {
+        lane_coeffs<A, PT, VEC, false>(p, l, w, b, sm_mu, sm_rs, nullptr, nullptr, sa, sb, unused1, unused2);
+        double_buffered(nb, issue, consume);
+      }
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
-        const A g = vd[j] * act_bwd<ACT, A>(vx[j] * sa[j] + sb[j]);
-        s1[j] += g * vx[j];
-        s2[j] += g;
+        sm1[l.ty * W + l.tx * VEC + j] = s1[j];
+        sm2[l.ty * W + l.tx * VEC + j] = s2[j];
       }
     }
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-      sm1[l.ty * W + l.tx * VEC + j] = s1[j];
-      sm2[l.ty * W + l.tx * VEC + j] = s2[j];
+    __syncthreads();
+    // per channel: sum the lane rows; keep gamma-weighted copies in row 0 for the group sums
+    for (int c = threadIdx.x; c < l.wch; c += kBlock) {
+      A t1 = (A)0, t2 = (A)0;
+      for (int ty = 0; ty < p.rpi; ++ty) {
+        t1 += sm1[ty * W + c];
+        t2 += sm2[ty * W + c];
+      }
+      const int64_t idx = ((n * p.tiles + l.tile) * p.C + l.cstart + c) * 2;
+      partC[idx] = t1;
+      partC[idx + 1] = t2;
+      const A gamma = w ? load_param<PT, A>(w, l.cstart + c) : (A)1;
+      sm1[c] = gamma * t1;
+      sm2[c] = gamma * t2;
     }
-  }
-  __syncthreads();
-  const int cstart = l.tc.chunk * p.lpr * VEC;
-  const int lanes_here = p.cv - l.tc.chunk * p.lpr < p.lpr ? p.cv - l.tc.chunk * p.lpr : p.lpr;
-  const int wch = lanes_here * VEC;
-  for (int c = threadIdx.x; c < wch; c += kBlock) {
-    A t1 = (A)0, t2 = (A)0;
-    for (int ety = 0; ety < p.rpi; ++ety) {
-      t1 += sm1[ety * W + c];
-      t2 += sm2[ety * W + c];
+    __syncthreads();
+    {
+      const int L = pow2_ceil_clamped(p.D < l.wch ? p.D : l.wch, 64);
+      const int nseg = kBlock / L;
+      const int seg = threadIdx.x / L, sl = threadIdx.x % L;
+      for (int base = 0; base < l.ng; base += nseg) {
+        const int gi = base + seg;
+        const int g = l.g_lo + gi;
+        const bool valid = gi < l.ng;
+        int ca = 0, cb = 0;
+        if (valid) group_span(p, l, g, ca, cb);
+        A ta = (A)0, tb = (A)0;
+        for (int c = ca + sl; c < cb; c += L) { ta += sm1[c]; tb += sm2[c]; }
+        ta = segment_sum(ta, L);
+        tb = segment_sum(tb, L);
+        if (valid && sl == 0) {
+          const int64_t slot = group_slot(q, p.G, n, l.tile, l.chunk, g);
+          partG[slot] = ta;
+          partG[plane + slot] = tb;
+        }
+      }
     }
-    const int64_t idx = ((l.tc.n * p.tiles + l.tc.tile) * p.C + cstart + c) * 2;
-    part[idx] = t1;
-    part[idx + 1] = t2;
+    __syncthreads();
   }
 }
 
+// Sum the tile partials (A, B) of group g with L lanes; every lane of the segment gets the sums.
+template <typename A>
+__device__ __forceinline__ void sum_group_partials(const A *__restrict__ partG, int64_t plane, const PartialGeo &q, int G,
+                                                   int D, int64_t n, int g, bool valid, int L, int sl, A &ta, A &tb) {
+  int k_lo = 0, nk = 1;
+  if (valid) group_chunks(q, D, g, k_lo, nk);
+  const int P = valid ? q.tiles * nk : 0;
+  const int64_t base = group_slot(q, G, n, 0, k_lo, g);
+  const int64_t kstride = (int64_t)G * q.tiles;
+  ta = (A)0;
+  tb = (A)0;
+  for (int e = sl; e < P; e += L) {
+    const int k = e / q.tiles, t = e - k * q.tiles;
+    const int64_t slot = base + k * kstride + t;
+    ta += partG[slot];
+    tb += partG[plane + slot];
+  }
+  ta = segment_sum(ta, L);
+  tb = segment_sum(tb, L);
+}
+
 // ---------------------------------------------------------------------------------------------
-// Backward pass 2, one workgroup per (n, g): sum the tile partials of the group's channels
-// (height_reduce, src/gnnhwc/csrc/gn_kernel.cu:648-693), then
-//   A = sum_c gamma_c S1_c, B = sum_c gamma_c S2_c, s = 1 / (D R),
-//   coef1 = (mean B - A) s rstd^3, coef2 = -mean coef1 - B s rstd
-// (compute_bwd_scale_biases, gn_kernel.cu:730-801).
-//   sums : [N][C][2]   coef : [N][G][2]
+// Optional backward pass 1b (many tiles per sample): sum the tile partials once.
+//   blocks [0, nG)      : one wavefront per (n, g)         -> outG 2 planes [N][G]
+//   blocks [nG, nG + nC): eight lanes per (n, c)           -> outC [N][C][2]   (height_reduce, gn_kernel.cu:648-693)
 // ---------------------------------------------------------------------------------------------
 template <typename A>
-__global__ __launch_bounds__(kBlock) void bwd_finalize_kernel(const A *__restrict__ part, const void *mean,
-                                                              const void *rstd, int sdtype, const void *w, int pdtype,
-                                                              A *__restrict__ sums, A *__restrict__ coef, Plan p) {
-  __shared__ A red[2 * (kBlock / 64)];
-  const int64_t n = blockIdx.x / p.G;
-  const int g = (int)(blockIdx.x - n * p.G);
-  int L = 1;
-  while (L < p.tiles && L < 64) L <<= 1;
-  const int per_pass = kBlock / L;
-  const int sub = threadIdx.x / L, sl = threadIdx.x % L;
-  A ga = (A)0, gb = (A)0;  // this thread's share of A and B (only segment leaders contribute)
-  for (int base = 0; base < p.D; base += per_pass) {
-    const int i = base + sub;
-    A s1 = (A)0, s2 = (A)0;
-    const int c = g * p.D + i;
-    if (i < p.D) {
-      for (int t = sl; t < p.tiles; t += L) {
-        const int64_t idx = ((n * p.tiles + t) * p.C + c) * 2;
-        s1 += part[idx];
-        s2 += part[idx + 1];
-      }
-    }
-    s1 = segment_sum(s1, L);
-    s2 = segment_sum(s2, L);
-    if (i < p.D && sl == 0) {
-      sums[(n * p.C + c) * 2] = s1;
-      sums[(n * p.C + c) * 2 + 1] = s2;
-      const A gamma = w ? load_scalar<A>(w, c, pdtype) : (A)1;
-      ga += gamma * s1;
-      gb += gamma * s2;
-    }
-  }
-  ga = segment_sum(ga, 64);
-  gb = segment_sum(gb, 64);
-  if ((threadIdx.x & 63) == 0) {
-    red[2 * (threadIdx.x >> 6)] = ga;
-    red[2 * (threadIdx.x >> 6) + 1] = gb;
-  }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    A ta = (A)0, tb = (A)0;
-    for (int wv = 0; wv < kBlock / 64; ++wv) { ta += red[2 * wv]; tb += red[2 * wv + 1]; }
-    const int64_t ng = n * p.G + g;
-    const A mu = load_scalar<A>(mean, ng, sdtype);
-    const A rs = load_scalar<A>(rstd, ng, sdtype);
-    const A s = (A)1 / ((A)p.D * (A)p.R);
-    const A c1 = (mu * tb - ta) * s * rs * rs * rs;
-    coef[ng * 2] = c1;
-    coef[ng * 2 + 1] = -mu * c1 - tb * s * rs;
-  }
-}
-
-// ---------------------------------------------------------------------------------------------
-// Backward pass 3: dx = a g + coef1 x + coef2 with g recomputed as in pass 1.  Does the work of
-// dx_elem_kernel (src/gnnhwc/csrc/gn_kernel.cu:803-905).  The last ceil(C / 256) workgroups of the grid
-// instead produce dgamma_c = sum_n (S1 - mean S2) rstd and dbeta_c = sum_n S2
-// (compute_dweight_dbias, gn_kernel.cu:695-728).
-// ---------------------------------------------------------------------------------------------
-template <typename T, int VEC, int ACT>
-__global__ __launch_bounds__(kBlock) void bwd_dx_kernel(const T *__restrict__ x, const T *__restrict__ dy,
-                                                        T *__restrict__ dx, const void *mean, const void *rstd,
-                                                        int sdtype, const void *w, const void *b, int pdtype,
-                                                        const acc_t<T> *__restrict__ sums,
-                                                        const acc_t<T> *__restrict__ coef, void *dw, void *db, Plan p) {
-  using A = acc_t<T>;
-  if ((int64_t)blockIdx.x >= p.nblocks) {
-    const int64_t c = ((int64_t)blockIdx.x - p.nblocks) * kBlock + threadIdx.x;
-    if (c < p.C) {
-      const int g = (int)(c / p.D);
-      A t1 = (A)0, t2 = (A)0;
-      for (int64_t n = 0; n < p.N; ++n) {
-        const A mu = load_scalar<A>(mean, n * p.G + g, sdtype);
-        const A rs = load_scalar<A>(rstd, n * p.G + g, sdtype);
-        const A s1 = sums[(n * p.C + c) * 2], s2 = sums[(n * p.C + c) * 2 + 1];
-        t1 += (s1 - mu * s2) * rs;
-        t2 += s2;
-      }
-      if (dw) store_scalar<A>(dw, c, pdtype, t1);
-      if (db) store_scalar<A>(db, c, pdtype, t2);
+__global__ __launch_bounds__(kBlock) void bwd_compact_kernel(const A *__restrict__ partC, const A *__restrict__ partG,
+                                                             A *__restrict__ outC, A *__restrict__ outG, PartialGeo q,
+                                                             int nG_blocks, Plan p) {
+  if ((int)blockIdx.x < nG_blocks) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int64_t item = (int64_t)blockIdx.x * (kBlock / 64) + wave;
+    const bool valid = item < p.N * p.G;
+    const int64_t n = valid ? item / p.G : 0;
+    const int g = valid ? (int)(item - n * p.G) : 0;
+    A ta, tb;
+    sum_group_partials<A>(partG, group_plane(q, p.G, p.N), q, p.G, p.D, n, g, valid, 64, lane, ta, tb);
+    if (valid && lane == 0) {
+      outG[item] = ta;
+      outG[p.N * p.G + item] = tb;
     }
     return;
   }
-  const LanePos l = lane_pos(p, true);
-  if (!l.active) return;
-  A sa[VEC], sb[VEC], c1[VEC], c2[VEC];
-  affine_coeffs<A, VEC>(p, l, mean, rstd, sdtype, w, b, pdtype, sa, sb);
-#pragma unroll
-  for (int j = 0; j < VEC; ++j) {
-    const int g = (l.cvi * VEC + j) / p.D;
-    c1[j] = coef[(l.tc.n * p.G + g) * 2];
-    c2[j] = coef[(l.tc.n * p.G + g) * 2 + 1];
-  }
-  const int64_t off = (l.tc.n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC;
-  const T *px = x + off;
-  const T *pdy = dy + off;
-  T *pdx = dx + off;
-  const int64_t step = (int64_t)p.rpi * p.C;
-  int lr = l.ty;
-  for (; lr + (kUnroll - 1) * p.rpi < l.len; lr += kUnroll * p.rpi) {
-    A vx[kUnroll][VEC], vd[kUnroll][VEC];
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      LaneVec<T, VEC, true>::load(px + u * step, vx[u]);
-      LaneVec<T, VEC, true>::load(pdy + u * step, vd[u]);
+  // channel sums: 32 channels per workgroup, 8 tile slices; consecutive lanes read consecutive channels
+  const int cl = threadIdx.x & 31, ts = threadIdx.x >> 5;
+  const int64_t nc = ((int64_t)blockIdx.x - nG_blocks) * 32 + cl;
+  __shared__ A red[2][8][32];
+  const bool valid = nc < p.N * p.C;
+  A t1 = (A)0, t2 = (A)0;
+  if (valid) {
+    const int64_t n = nc / p.C, c = nc - n * p.C;
+    for (int t = ts; t < q.tiles; t += 8) {
+      const int64_t idx = ((n * q.tiles + t) * p.C + c) * 2;
+      t1 += partC[idx];
+      t2 += partC[idx + 1];
     }
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        const A g = vd[u][j] * act_bwd<ACT, A>(vx[u][j] * sa[j] + sb[j]);
-        vd[u][j] = sa[j] * g + (c1[j] * vx[u][j] + c2[j]);
+  }
+  red[0][ts][cl] = t1;
+  red[1][ts][cl] = t2;
+  __syncthreads();
+  if (valid && ts == 0) {
+    A r1 = (A)0, r2 = (A)0;
+    for (int s = 0; s < 8; ++s) { r1 += red[0][s][cl]; r2 += red[1][s][cl]; }
+    outC[nc * 2] = r1;
+    outC[nc * 2 + 1] = r2;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Backward pass 2: sum the tile partials A, B of the chunk's groups, s = 1 / (D R),
+//   coef1 = (mean B - A) s rstd^3, coef2 = -mean coef1 - B s rstd      (gn_kernel.cu:798-800)
+//   dx = a g + coef1 x + coef2, g recomputed as in pass 1                (dx_elem_kernel, gn_kernel.cu:803-905)
+// One extra column of workgroups (blockIdx.x == tiles, sample 0 only) produces, for the channels of its
+// chunk, dgamma_c = sum_n (S1 - mean S2) rstd and dbeta_c = sum_n S2 (compute_dweight_dbias, gn_kernel.cu:695-728).
+// ---------------------------------------------------------------------------------------------
+template <typename T, typename PT, int VEC, int ACT>
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) void bwd_dx_kernel(
+    const T *__restrict__ x, const T *__restrict__ dy, T *__restrict__ dx, const void *mean, const void *rstd, int sdtype,
+    const void *w, const void *b, const acc_t<T> *__restrict__ partC, const acc_t<T> *__restrict__ partG, PartialGeo q,
+    void *dw, void *db, Plan p) {
+  using A = acc_t<T>;
+  using LV = LaneVec<T, VEC>;
+  constexpr int U = kUnrollBwd;
+  __shared__ A sm_c1[kBlock * VEC];
+  __shared__ A sm_c2[kBlock * VEC];
+  __shared__ A sm_mu[kBlock * VEC];
+  __shared__ A sm_rs[kBlock * VEC];
+  if ((int)blockIdx.x == p.tiles) {
+    if (blockIdx.z != 0 || (!dw && !db)) return;
+    const int cstart = blockIdx.y * p.lpr * p.vec;
+    const int lanes_here = p.cv - (int)blockIdx.y * p.lpr < p.lpr ? p.cv - (int)blockIdx.y * p.lpr : p.lpr;
+    const int wch = lanes_here * p.vec;
+    // threads are laid out (tile slice, channel): consecutive threads read consecutive channels
+    const int cw = wch < kBlock ? wch : kBlock;  // channels handled per pass
+    const int nsl = kBlock / cw;                 // tile slices
+    const int cl = threadIdx.x % cw, ts = threadIdx.x / cw;
+    for (int cbase = 0; cbase < wch; cbase += cw) {
+      const int c = cstart + cbase + cl;
+      A t1 = (A)0, t2 = (A)0;
+      if (cbase + cl < wch && ts < nsl) {
+        const int g = c / p.D;
+        for (int64_t n = 0; n < p.N; ++n) {
+          A s1 = (A)0, s2 = (A)0;
+          for (int t = ts; t < q.tiles; t += nsl) {
+            const int64_t idx = ((n * q.tiles + t) * p.C + c) * 2;
+            s1 += partC[idx];
+            s2 += partC[idx + 1];
+          }
+          const A mu = load_scalar<A>(mean, n * p.G + g, sdtype);
+          const A rs = load_scalar<A>(rstd, n * p.G + g, sdtype);
+          t1 += (s1 - mu * s2) * rs;
+          t2 += s2;
+        }
       }
-      LaneVec<T, VEC, true>::store(pdx + u * step, vd[u]);
+      __syncthreads();
+      if (ts < nsl) { sm_c1[ts * cw + cl] = t1; sm_c2[ts * cw + cl] = t2; }
+      __syncthreads();
+      if (ts == 0 && cbase + cl < wch) {
+        A r1 = (A)0, r2 = (A)0;
+        for (int s = 0; s < nsl; ++s) { r1 += sm_c1[s * cw + cl]; r2 += sm_c2[s * cw + cl]; }
+        if (dw) store_param<PT, A>(dw, c, r1);
+        if (db) store_param<PT, A>(db, c, r2);
+      }
     }
-    px += kUnroll * step;
-    pdy += kUnroll * step;
-    pdx += kUnroll * step;
+    return;
   }
-  for (; lr < l.len; lr += p.rpi) {
-    A vx[VEC], vd[VEC];
-    LaneVec<T, VEC, true>::load(px, vx);
-    LaneVec<T, VEC, true>::load(pdy, vd);
+  const int64_t plane = group_plane(q, p.G, p.N);
+  for (int64_t n = blockIdx.z; n < p.N; n += gridDim.z) {
+    const LanePos l = lane_pos(p, n, true);
+    const int rows = l.rows;
+    const int nb = (rows + U - 1) / U;
+    const int64_t off = (n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC;
+    const int64_t step = (int64_t)p.rpi * p.C;
+    typename LV::raw_t bx0[U], bx1[U], bd0[U], bd1[U];
+    A sa[VEC], sb[VEC], c1[VEC], c2[VEC];
+    auto issue = [&](auto sel, int bi) {
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-      const A g = vd[j] * act_bwd<ACT, A>(vx[j] * sa[j] + sb[j]);
-      vd[j] = sa[j] * g + (c1[j] * vx[j] + c2[j]);
+      for (int u = 0; u < U; ++u) {
+        const int64_t o = off + (int64_t)clamp_row(bi * U + u, rows) * step;
+        if constexpr (decltype(sel)::value == 0) { bx0[u] = LV::load(x + o); bd0[u] = LV::load(dy + o); }
+        else { bx1[u] = LV::load(x + o); bd1[u] = LV::load(dy + o); }
+      }
+    };
+    auto consume = [&](auto sel, int bi) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        A vx[VEC], vd[VEC];
+        if constexpr (decltype(sel)::value == 0) { LV::unpack(bx0[u], vx); LV::unpack(bd0[u], vd); }
+        else { LV::unpack(bx1[u], vx); LV::unpack(bd1[u], vd); }
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const A g = vd[j] * act_bwd<ACT, A>(vx[j] * sa[j] + sb[j]);
+          vd[j] = sa[j] * g + (c1[j] * vx[j] + c2[j]);
+        }
+        LV::store(dx + off + (int64_t)clamp_row(bi * U + u, rows) * step, LV::pack(vd));
+      }
+    };
+    if (nb > 0) issue(std::integral_constant<int, 0>{}, 0);  // in flight while the group sums are merged
+    {
+      const int L = merge_lanes(q, p.D);
+      const int nseg = kBlock / L;
+      const int seg = threadIdx.x / L, sl = threadIdx.x % L;
+      for (int base = 0; base < l.ng; base += nseg) {
+        const int gi = base + seg;
+        const bool valid = gi < l.ng;
+        const int g = l.g_lo + gi;
+        A ta, tb;
+        sum_group_partials<A>(partG, plane, q, p.G, p.D, n, g, valid, L, sl, ta, tb);
+        if (valid && sl == 0) {
+          const A mu = load_scalar<A>(mean, n * p.G + g, sdtype);
+          const A rs = load_scalar<A>(rstd, n * p.G + g, sdtype);
+          const A s = (A)1 / ((A)p.D * (A)p.R);
+          const A k1 = (mu * tb - ta) * s * rs * rs * rs;
+          sm_mu[gi] = mu;
+          sm_rs[gi] = rs;
+          sm_c1[gi] = k1;
+          sm_c2[gi] = -mu * k1 - tb * s * rs;
+        }
+      }
     }
-    LaneVec<T, VEC, true>::store(pdx, vd);
-    px += step;
-    pdy += step;
-    pdx += step;
+    __syncthreads();
+    if (nb > 0) {
+      lane_coeffs<A, PT, VEC, true>(p, l, w, b, sm_mu, sm_rs, sm_c1, sm_c2, sa, sb, c1, c2);
+      double_buffered(nb, issue, consume);
+    }
+    __syncthreads();
   }
 }
 

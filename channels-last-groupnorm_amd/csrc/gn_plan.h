@@ -10,15 +10,18 @@ namespace gn {
 enum { GN_F32 = 0, GN_F64 = 1, GN_F16 = 2, GN_BF16 = 3 };
 enum { GN_ACT_IDENTITY = 0, GN_ACT_RELU = 1, GN_ACT_SILU = 2, GN_ACT_GELU = 3, GN_ACT_GELU_TANH = 4 };
 
-constexpr int kBlock = 256;    // threads per workgroup (4 wavefronts)
-constexpr int kUnroll = 4;     // independent row loads in flight per lane
-constexpr int kNumCU = 256;    // MI355X
-constexpr int kTargetBlocks = 2048;  // aim for ~8 workgroups per CU when the tensor is large enough
+constexpr int kBlock = 256;         // threads per workgroup (4 wavefronts)
+constexpr int kUnrollFwd = 4;       // independent row loads in flight per lane, one-input kernels
+constexpr int kUnrollBwd = 2;       // ... two-input kernels (x and dy)
+constexpr int kNumCU = 256;         // MI355X
+constexpr int kTargetBlocks = 512;  // aim for ~2 workgroups per CU when the tensor is large enough
+constexpr int kMaxInlineEntries = 2048;  // tile partials a consumer workgroup may merge in its prologue
 
 // One workgroup owns `tile_rows` consecutive rows of one sample and one chunk of `lpr` lane vectors
 // (lpr * vec channels) of every such row.  Inside the workgroup thread t handles lane vector
 // (t % lpr) of rows (t / lpr), (t / lpr) + rpi, ...: every lane keeps the same channels for the whole
 // tile, so per-channel affine coefficients and per-channel partial sums live in registers.
+// Grid: x = row tile, y = channel chunk, z = sample (z wraps when N exceeds the grid limit).
 struct Plan {
   int64_t N, R, C;
   int G, D;         // groups, channels per group
@@ -29,7 +32,15 @@ struct Plan {
   int rpi;          // rows covered per step = kBlock / lpr
   int tile_rows;    // rows per workgroup tile
   int tiles;        // row tiles per sample = ceil(R / tile_rows)
+  int gmax;         // most groups any chunk intersects
   int64_t nblocks;  // N * tiles * nchunk
+};
+
+// Geometry of a buffer of per-tile partial results as the consumer sees it: either the producer's own
+// (tiles, nchunk), or (1, 1) after the compaction kernel has merged all tiles of a sample.
+struct PartialGeo {
+  int tiles, nchunk;
+  int chunk_channels;  // channels per chunk of the producer (lpr * vec); C when compacted
 };
 
 }  // namespace gn

@@ -1,0 +1,77 @@
+"""Helpers for the GPU parity tests: direct calls through the C ABI on torch-owned device memory, and the
+error metrics the tolerances are written in."""
+import ctypes
+
+import numpy as np
+import torch
+
+from gnnhwc import _cabi
+
+DT_CODE = {torch.float32: 0, torch.float64: 1, torch.float16: 2, torch.bfloat16: 3}
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def nrc_view(t):
+    """(N, C, *spatial) tensor with channels fastest -> (N, R, C) contiguous tensor (no copy when already laid out so)."""
+    nd = t.dim()
+    u = t.permute(0, *range(2, nd), 1)
+    u = u if u.is_contiguous() else u.contiguous()
+    return u.reshape(u.shape[0], -1, u.shape[-1])
+
+
+def cabi_fwd(x_nrc, w, b, G, eps, act, stats_dtype=None, y=None, ws=None):
+    """gnnhwc_fwd on (N, R, C) device tensors.  Returns y, mean, rstd."""
+    N, R, C = x_nrc.shape
+    dt = DT_CODE[x_nrc.dtype]
+    sdtype = stats_dtype or (torch.float32 if x_nrc.dtype in (torch.float16, torch.bfloat16) else x_nrc.dtype)
+    pdt = DT_CODE[w.dtype] if w is not None else dt
+    y = torch.empty_like(x_nrc) if y is None else y
+    mean = torch.empty((N, G), dtype=sdtype, device=x_nrc.device)
+    rstd = torch.empty((N, G), dtype=sdtype, device=x_nrc.device)
+    lib = _cabi.lib
+    nbytes = lib.gnnhwc_fwd_workspace_bytes(N, R, C, G, dt)
+    assert nbytes > 0, _cabi.last_error()
+    ws = torch.empty((nbytes,), dtype=torch.uint8, device=x_nrc.device) if ws is None else ws
+    rc = lib.gnnhwc_fwd(_ptr(x_nrc), _ptr(w), _ptr(b), _ptr(y), _ptr(mean), _ptr(rstd), N, R, C, G, float(eps), int(act),
+                        dt, pdt, DT_CODE[sdtype], _ptr(ws), ws.numel(), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    _cabi.check(rc, "gnnhwc_fwd")
+    return y, mean, rstd
+
+
+def cabi_bwd(dy_nrc, x_nrc, w, b, mean, rstd, G, act, dx=None, ws=None, want_dw=True, want_db=True):
+    N, R, C = x_nrc.shape
+    dt = DT_CODE[x_nrc.dtype]
+    pdtype = w.dtype if w is not None else x_nrc.dtype
+    dx = torch.empty_like(x_nrc) if dx is None else dx
+    dw = torch.empty((C,), dtype=pdtype, device=x_nrc.device) if want_dw else None
+    db = torch.empty((C,), dtype=pdtype, device=x_nrc.device) if want_db else None
+    lib = _cabi.lib
+    nbytes = lib.gnnhwc_bwd_workspace_bytes(N, R, C, G, dt)
+    assert nbytes > 0, _cabi.last_error()
+    ws = torch.empty((nbytes,), dtype=torch.uint8, device=x_nrc.device) if ws is None else ws
+    rc = lib.gnnhwc_bwd(_ptr(dy_nrc), _ptr(x_nrc), _ptr(w), _ptr(b), _ptr(mean), _ptr(rstd), _ptr(dx), _ptr(dw), _ptr(db),
+                        N, R, C, G, int(act), dt, DT_CODE[pdtype], DT_CODE[mean.dtype], _ptr(ws), ws.numel(),
+                        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    _cabi.check(rc, "gnnhwc_bwd")
+    return dx, dw, db
+
+
+def err(a, truth):
+    """max_i |a_i - t_i| / (|t_i| + rms(t)): relative for elements of typical size, and relative to the
+    tensor's scale for elements near zero (where a pure ratio is meaningless)."""
+    a = torch.as_tensor(a).detach().to("cpu", torch.float64).reshape(-1)
+    t = torch.as_tensor(truth).detach().to("cpu", torch.float64).reshape(-1)
+    assert a.shape == t.shape, (a.shape, t.shape)
+    if t.numel() == 0:
+        return 0.0
+    rms = float(t.square().mean().sqrt())
+    if rms == 0.0:
+        rms = 1.0
+    return float(((a - t).abs() / (t.abs() + rms)).max())
+
+
+def as_np64(t):
+    return t.detach().to("cpu", torch.float64).numpy()

@@ -1,0 +1,93 @@
+"""GPU parity: the HIP path, called through the C ABI, against the CPU oracle (oracle/gn_oracle.c in float64)
+and against torch's own GroupNorm + activation on the same seeded inputs.
+
+Tolerances (the build's stated bar):
+  fp32 / fp64 : err <= 1e-5 (fp64: 1e-12), with err = max |ours - truth| / (|truth| + rms(truth));
+  fp16 / bf16 : err(ours vs float64 truth) <= err(torch's own fp16/bf16 GroupNorm+activation vs the same truth)
+                times (1 + HALF_SLACK) -- i.e. no worse than the library routine's own half-precision error.
+relu's derivative is discontinuous at 0: dx elements whose pre-activation is within RELU_BAND of 0 are
+left out of the element-wise comparison (they may legitimately land on either side).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gn_oracle as orc
+from tests import configs
+from tests.gpu_harness import as_np64, cabi_bwd, cabi_fwd, err, nrc_view
+
+pytestmark = pytest.mark.gpu
+
+FP32_TOL = 1e-5
+FP64_TOL = 1e-12
+HALF_SLACK = 0.02
+RELU_BAND = 1e-4
+EPS = 1e-5
+
+
+def _truth(inp, G, act_code):
+    x = as_np64(nrc_view(inp["x"]))
+    dy = as_np64(nrc_view(inp["dy"]))
+    return orc.fwd_bwd(x, as_np64(inp["w"]), as_np64(inp["b"]), dy, G, EPS, act_code)
+
+
+def _torch_same_dtype(inp, G, act):
+    """torch's GroupNorm + activation + autograd on the device, in the inputs' own dtype."""
+    r = orc.torch_reference(inp["x"], inp["w"], inp["b"], G, EPS, act, inp["dy"])
+    return {"y": as_np64(nrc_view(r["y"])), "dx": as_np64(nrc_view(r["dx"])), "dw": as_np64(r["dw"]), "db": as_np64(r["db"])}
+
+
+def _relu_mask(inp, truth, G):
+    x = as_np64(nrc_view(inp["x"]))
+    N, R, C = x.shape
+    D = C // G
+    a = np.repeat(truth["rstd"], D, axis=1) * as_np64(inp["w"])[None, :]
+    b = as_np64(inp["b"])[None, :] - np.repeat(truth["mean"], D, axis=1) * a
+    z = x * a[:, None, :] + b[:, None, :]
+    return np.abs(z) > RELU_BAND
+
+
+def _check(name, ours, truth, lib_result, dtype, mask=None):
+    o, t = as_np64(ours) if isinstance(ours, torch.Tensor) else ours, truth
+    if mask is not None:
+        o, t = np.where(mask, o, 0.0), np.where(mask, t, 0.0)
+    e = err(o, t)
+    if dtype == torch.float32:
+        assert e <= FP32_TOL, "%s: err %.3g > %.1g" % (name, e, FP32_TOL)
+    elif dtype == torch.float64:
+        assert e <= FP64_TOL, "%s: err %.3g > %.1g" % (name, e, FP64_TOL)
+    else:
+        l = lib_result if mask is None else np.where(mask, lib_result, 0.0)
+        e_lib = err(l, t)
+        assert e <= e_lib * (1 + HALF_SLACK), "%s: err %.3g vs torch's own %s error %.3g" % (name, e, dtype, e_lib)
+    return e
+
+
+@pytest.mark.parametrize("name", configs.ALL_NAMES)
+def test_config_parity(name, device):
+    cfg = configs.CONFIGS[name]
+    print("config", name, cfg, flush=True)
+    inp = configs.make_inputs(cfg, device)
+    act = orc.ACT_CODES[cfg.act]
+    dtype = configs.DT[cfg.dtype]
+    x, dy = nrc_view(inp["x"]), nrc_view(inp["dy"])
+    truth = _truth(inp, cfg.G, act)
+    lib = _torch_same_dtype(inp, cfg.G, cfg.act) if dtype in (torch.float16, torch.bfloat16) else None
+    y, mean, rstd = cabi_fwd(x, inp["w"], inp["b"], cfg.G, EPS, act)
+    torch.cuda.synchronize()
+    _check("mean", mean, truth["mean"], None, torch.float32 if dtype != torch.float64 else dtype)
+    _check("rstd", rstd, truth["rstd"], None, torch.float32 if dtype != torch.float64 else dtype)
+    _check("y", y, truth["y"], lib and lib["y"], dtype)
+    if cfg.passes == "fwd":
+        return
+    dx, dw, db = cabi_bwd(dy, x, inp["w"], inp["b"], mean, rstd, cfg.G, act)
+    torch.cuda.synchronize()
+    mask = _relu_mask(inp, truth, cfg.G) if cfg.act == "relu" else None
+    _check("dx", dx, truth["dx"], lib and lib["dx"], dtype, mask)
+    _check("dw", dw, truth["dw"], lib and lib["dw"], dtype)
+    _check("db", db, truth["db"], lib and lib["db"], dtype)
+    # size-independent property: dx sums to zero over every (n, g) slab, relative to the slab's absolute sum
+    N, R, C = x.shape
+    slab = as_np64(dx).reshape(N, R, cfg.G, C // cfg.G)
+    ulp = {torch.float32: 2.0 ** -24, torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}[dtype]
+    assert np.max(np.abs(slab.sum(axis=(1, 3))) / np.abs(slab).sum(axis=(1, 3))) < 4 * ulp
