@@ -5,6 +5,9 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <time.h>
+
+#include <atomic>
 #include <vector>
 
 #include "../../include/gnnhwc.h"
@@ -142,23 +145,29 @@ int check_dtypes(int dtype, int pdtype, int sdtype) {
 bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 size_t acc_size(int dtype) { return dtype == GN_F64 ? 8 : 4; }
+size_t max_size(size_t a, size_t b) { return a > b ? a : b; }
 size_t fwd_ws_bytes(int64_t N, int64_t R, int64_t C, int64_t G, int dtype) {
   const int vec = 16 / elem_size(dtype);
   size_t need = fwd_workspace(make_plan(N, R, C, G, 1, 1)).total;
+  size_t resident = 0;
   if (C % vec == 0) {
     const size_t v = fwd_workspace(make_plan(N, R, C, G, vec, 1)).total;
     if (v > need) need = v;
+    resident = dtype == GN_F64 ? 0 : resident_fwd_bytes(G);
   }
-  return need * acc_size(dtype);
+  return max_size(need * acc_size(dtype), resident);
 }
 size_t bwd_ws_bytes(int64_t N, int64_t R, int64_t C, int64_t G, int dtype) {
   const int vec = 16 / elem_size(dtype);
   size_t need = bwd_workspace(make_plan(N, R, C, G, 1, 2)).total;
+  size_t resident = 0;
   if (C % vec == 0) {
-    const size_t v = bwd_workspace(make_plan(N, R, C, G, vec, 2)).total;
+    const Plan pv = make_plan(N, R, C, G, vec, 2);
+    const size_t v = bwd_workspace(pv).total;
     if (v > need) need = v;
+    resident = dtype == GN_F64 ? 0 : resident_bwd_bytes((int64_t)pv.lpr * vec, G);
   }
-  return need * acc_size(dtype);
+  return max_size(need * acc_size(dtype), resident);
 }
 
 __global__ void fill_zero_kernel(void *p, int64_t n, int dtype) {
@@ -192,6 +201,33 @@ hipEvent_t get_event() {
 }
 
 }  // namespace
+
+unsigned long long next_epoch() {
+  static std::atomic<unsigned long long> counter{0};
+  static const unsigned long long seed = []() {
+    unsigned long long v = (unsigned long long)time(nullptr) * 0x9E3779B97F4A7C15ull;
+    v ^= (unsigned long long)(uintptr_t)&counter << 17;
+    return v | 1ull;
+  }();
+  // odd multiplier: distinct counters give distinct epochs; never 0
+  unsigned long long e = seed + 0x9E3779B97F4A7C15ull * (counter.fetch_add(1) + 1);
+  return e ? e : 1ull;
+}
+unsigned long long *trace_buffer() {
+  static unsigned long long *buf = []() -> unsigned long long * {
+    if (env_int("GNNHWC_TRACE", 0) == 0) return nullptr;
+    void *p = nullptr;
+    const size_t bytes = (size_t)kMaxResidentBlocks * 8 * sizeof(unsigned long long);
+    if (hipMalloc(&p, bytes) != hipSuccess) return nullptr;
+    (void)hipMemset(p, 0, bytes);
+    return (unsigned long long *)p;
+  }();
+  return buf;
+}
+bool resident_enabled() {
+  static const int off = env_int("GNNHWC_DISABLE_RESIDENT", 0);
+  return off == 0;
+}
 
 void profile_before(int kind, hipStream_t stream) {
   if (!g_profile) return;
@@ -332,6 +368,16 @@ int gnnhwc_profile_collect(int64_t *launches, double *total_ms) {
   }
   g_timed.clear();
   return rc;
+}
+
+int gnnhwc_debug_read_trace(unsigned long long *out, int64_t count) {
+  unsigned long long *buf = trace_buffer();
+  if (!buf) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "tracing is off (set GNNHWC_TRACE=1 before the first call)");
+  const int64_t cap = (int64_t)kMaxResidentBlocks * 8;
+  if (!out || count <= 0 || count > cap) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "trace read of %lld words (capacity %lld)", (long long)count, (long long)cap);
+  const hipError_t e = hipMemcpy(out, buf, (size_t)count * sizeof(unsigned long long), hipMemcpyDeviceToHost);
+  if (e != hipSuccess) return fail(GNNHWC_ERR_LAUNCH, "trace read failed: %s", hipGetErrorString(e));
+  return GNNHWC_OK;
 }
 
 const char *gnnhwc_kernel_kind_name(int kind) {

@@ -207,7 +207,10 @@ template <int ACT, typename A> __device__ __forceinline__ A act_bwd(A z) {
 // correction 0, gn_kernel.cu:175,254).  Where the reference merges triples pairwise with
 // WelfordOps::combine (Welford.h:44-65), sets of triples are merged here with the equivalent exact
 // two-pass form, which is a pair of plain sums and therefore reduces with fixed butterfly trees:
-//   n = sum n_i,  mean = sum n_i mean_i / n,  M2 = sum (M2_i + n_i (mean_i - mean)^2).
+//   n = sum n_i,  mean = sum n_i mean_i / n,  M2 = sum (M2_i + n_i (mean_i - mean)^2),
+// or, where one pass must do, with the same sums taken about a pivot K that is itself the mean of one of
+// the parts (so |K - mean| is a small fraction of the spread and nothing cancels):
+//   s1 = sum n_i (mean_i - K),  s2 = sum (M2_i + n_i (mean_i - K)^2),  mean = K + s1 / n,  M2 = s2 - s1^2 / n.
 // ---------------------------------------------------------------------------------------------
 template <typename A> struct Moments {
   A n, mean, m2;
@@ -215,11 +218,51 @@ template <typename A> struct Moments {
 template <typename A> __device__ __forceinline__ A shfl_xor_acc(A v, int mask, int width) {
   return __shfl_xor(v, mask, width);
 }
-// Butterfly sum over `width` consecutive lanes (power of two <= 64).  Every lane of the segment ends with
-// the same bits: the tree is fixed and floating-point addition is commutative.
+// Cross-lane exchange inside a row of 16 lanes with a DPP modifier (VALU latency, no LDS traffic).
+template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
+  const int i = __builtin_bit_cast(int, v);
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(i, i, CTRL, 0xF, 0xF, false));
+}
+template <int CTRL> __device__ __forceinline__ double dpp_move(double v) {
+  const unsigned long long u = __builtin_bit_cast(unsigned long long, v);
+  const int lo = (int)(unsigned)u, hi = (int)(unsigned)(u >> 32);
+  const unsigned rlo = (unsigned)__builtin_amdgcn_update_dpp(lo, lo, CTRL, 0xF, 0xF, false);
+  const unsigned rhi = (unsigned)__builtin_amdgcn_update_dpp(hi, hi, CTRL, 0xF, 0xF, false);
+  return __builtin_bit_cast(double, (unsigned long long)rlo | ((unsigned long long)rhi << 32));
+}
+constexpr int kDppQuadXor1 = 0xB1;       // quad_perm:[1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;       // quad_perm:[2,3,0,1]
+constexpr int kDppRowHalfMirror = 0x141; // lane i <-> 7 - i inside each 8
+constexpr int kDppRowMirror = 0x140;     // lane i <-> 15 - i inside each 16
+// Sum over `width` consecutive lanes (power of two <= 64, aligned).  Every lane of the segment ends with
+// the same bits: each step adds the value of a lane from the other half of the growing group, whose
+// members already agree, and floating-point addition is commutative.  The first four steps are DPP
+// moves; only widths 32 and 64 need a trip through the LDS crossbar.
 template <typename A> __device__ __forceinline__ A segment_sum(A v, int width) {
-  for (int off = width >> 1; off > 0; off >>= 1) v += shfl_xor_acc(v, off, width);
+  if (width >= 2) v += dpp_move<kDppQuadXor1>(v);
+  if (width >= 4) v += dpp_move<kDppQuadXor2>(v);
+  if (width >= 8) v += dpp_move<kDppRowHalfMirror>(v);
+  if (width >= 16) v += dpp_move<kDppRowMirror>(v);
+  if (width >= 32) v += shfl_xor_acc(v, 16, 64);
+  if (width >= 64) v += shfl_xor_acc(v, 32, 64);
   return v;
+}
+// Two independent sums at once (their latencies overlap).
+template <typename A> __device__ __forceinline__ void segment_sum2(A &a, A &b, int width) {
+  if (width >= 2) { a += dpp_move<kDppQuadXor1>(a); b += dpp_move<kDppQuadXor1>(b); }
+  if (width >= 4) { a += dpp_move<kDppQuadXor2>(a); b += dpp_move<kDppQuadXor2>(b); }
+  if (width >= 8) { a += dpp_move<kDppRowHalfMirror>(a); b += dpp_move<kDppRowHalfMirror>(b); }
+  if (width >= 16) { a += dpp_move<kDppRowMirror>(a); b += dpp_move<kDppRowMirror>(b); }
+  if (width >= 32) {
+    const A oa = shfl_xor_acc(a, 16, 64), ob = shfl_xor_acc(b, 16, 64);
+    a += oa;
+    b += ob;
+  }
+  if (width >= 64) {
+    const A oa = shfl_xor_acc(a, 32, 64), ob = shfl_xor_acc(b, 32, 64);
+    a += oa;
+    b += ob;
+  }
 }
 __device__ __forceinline__ int pow2_ceil_clamped(int v, int hi) {
   int p = 1;

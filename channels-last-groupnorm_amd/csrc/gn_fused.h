@@ -1,0 +1,475 @@
+// Single-launch ("resident") GroupNorm kernels: the whole activation tensor is held in the register
+// files of the workgroups of one launch, so x (and dy) are read from memory exactly once.
+//
+//   forward : load tile -> per-tile group moments -> publish -> wait for the tiles that share my
+//             groups -> merge -> y = act(x a + b) from registers
+//   backward: load tile (x, dy) -> per-tile channel / group sums -> publish -> wait -> merge ->
+//             dx from registers; the workgroups of row tile 0 of sample 0 also finish dgamma / dbeta
+//
+// The launch must be small enough for every workgroup to be resident at once (the host checks this
+// against the occupancy the runtime reports and otherwise uses the streaming kernels): a workgroup
+// spins on data written by other workgroups of the same launch.
+//
+// Exchange protocol.  The XCDs' L2 caches are not coherent with each other, and the fences that would
+// make ordinary stores visible across them (L2 write-back / invalidate) cost tens of microseconds when
+// every workgroup issues them.  So everything that crosses workgroups is written with device-scope
+// (write-through) stores and read with device-scope (cache-bypassing) loads, and no fence is used.
+//  * Per-group tile results travel as 16-byte records {value0, value1, epoch (64 bit)} written by a
+//    single 128-bit store and read by a single 128-bit load: a consumer that sees this call's epoch in a
+//    record has the values that were stored with it.  The epoch is a fresh 64-bit value per call, so
+//    the workspace never needs clearing.  One memory round trip carries both "ready" and the data.
+//  * Per-channel sums for dgamma / dbeta use a flag per workgroup: every wave waits for the
+//    acknowledgement of its device-scope stores (s_waitcnt 0), the workgroup barriers, one thread
+//    stores the flag; the consumer loads the data only after it has seen the flag.
+// Polling is bounded by kMaxSpins; a timeout only records the epoch in a status word, so the grid
+// always drains.  Only fp32-accumulating element types use these kernels (a record has room for two
+// 32-bit values); float64 data takes the streaming kernels.
+#pragma once
+#include "gn_kernels.h"
+
+namespace gn {
+
+constexpr int kMaxSpins = 1 << 22;
+constexpr int kRecFast = 4;
+constexpr int kMaxResidentBlocksDev = 4 * kNumCU;  // records a lane keeps in registers while polling
+
+struct SyncArea {
+  void *recs;                 // 16-byte records, laid out [N][nchunk][G][tiles]
+  unsigned rec_bytes;
+  unsigned long long *flags;  // [N][nchunk][tiles]
+  unsigned long long epoch;   // value that marks "written in this call"
+  unsigned long long *status; // set to the epoch if a wait of this call timed out
+  unsigned long long *trace;  // optional [workgroup][kTracePoints] timestamps (100 MHz wall clock), else null
+};
+constexpr int kTracePoints = 8;
+__device__ __forceinline__ void trace_point(const SyncArea &s, int point) {
+  if (s.trace) __builtin_amdgcn_s_waitcnt(0);  // stamp a phase only once its memory operations have completed
+  if (s.trace && threadIdx.x == 0) {
+    const int64_t b = ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+    if (b < kMaxResidentBlocksDev) s.trace[b * kTracePoints + point] = wall_clock64();
+  }
+}
+
+__device__ __forceinline__ int64_t flag_index(const Plan &p, int64_t n, int k, int t) {
+  return (n * p.nchunk + k) * p.tiles + t;
+}
+
+// 128-bit device-scope accesses through a raw buffer descriptor (cache policy sc1)
+constexpr int kAuxDeviceScope = 16;
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t record_buffer(const SyncArea &s) {
+  return __builtin_amdgcn_make_buffer_rsrc(s.recs, 0, (int)s.rec_bytes, 0x27000);
+}
+__device__ __forceinline__ void record_store(__amdgpu_buffer_rsrc_t r, int64_t idx, float v0, float v1,
+                                             unsigned long long epoch) {
+  const u32x4 rec = {__builtin_bit_cast(unsigned, v0), __builtin_bit_cast(unsigned, v1), (unsigned)epoch,
+                     (unsigned)(epoch >> 32)};
+  __builtin_amdgcn_raw_buffer_store_b128(rec, r, (int)(idx * 16), 0, kAuxDeviceScope);
+}
+__device__ __forceinline__ u32x4 record_load(__amdgpu_buffer_rsrc_t r, int64_t idx) {
+  return __builtin_amdgcn_raw_buffer_load_b128(r, (int)(idx * 16), 0, kAuxDeviceScope);
+}
+__device__ __forceinline__ bool record_ready(const u32x4 &rec, unsigned long long epoch) {
+  return rec.z == (unsigned)epoch && rec.w == (unsigned)(epoch >> 32);
+}
+
+// Elements behind record (tile t, chunk k, group g): the rows of the tile times the channels of g in chunk k.
+__device__ __forceinline__ float record_count(const Plan &p, int t, int k, int g) {
+  const int cc = p.lpr * p.vec;
+  const int64_t c_lo = (int64_t)g * p.D > (int64_t)k * cc ? (int64_t)g * p.D : (int64_t)k * cc;
+  int64_t c_hi = (int64_t)(g + 1) * p.D < (int64_t)(k + 1) * cc ? (int64_t)(g + 1) * p.D : (int64_t)(k + 1) * cc;
+  if (c_hi > p.C) c_hi = p.C;
+  const int64_t rem = p.R - (int64_t)t * p.tile_rows;
+  const int64_t rows = rem < p.tile_rows ? rem : p.tile_rows;
+  return (float)((c_hi - c_lo) * rows);
+}
+
+// Collect the records of group g (all tiles of the chunks that hold a piece of it) with L lanes and reduce
+// them with reduce(e0[], e1[], cnt[], n_mine): each lane polls its own records until they carry this call's
+// epoch.  Up to kRecFast records per lane stay in registers (one round trip); more are polled first and
+// then re-read.  Returns through `out` whatever reduce produces from (value0, value1, count) per record.
+template <typename BODY>
+__device__ __forceinline__ void for_group_records(const SyncArea &s, __amdgpu_buffer_rsrc_t rb, const PartialGeo &q,
+                                                  const Plan &p, int64_t n, int g, bool valid, int L, int sl, BODY &&body) {
+  int k_lo = 0, nk = 1;
+  if (valid) group_chunks(q, p.D, g, k_lo, nk);
+  const int P = valid ? q.tiles * nk : 0;
+  const int64_t base = group_slot(q, p.G, n, 0, k_lo, g);
+  const int64_t kstride = (int64_t)p.G * q.tiles;
+  int spins = 0;
+  for (int e0 = sl; e0 < P; e0 += kRecFast * L) {
+    u32x4 rec[kRecFast];
+    bool have[kRecFast];
+    int64_t idx[kRecFast];
+    int kk[kRecFast], tt[kRecFast];
+#pragma unroll
+    for (int i = 0; i < kRecFast; ++i) {
+      const int e = e0 + i * L;
+      have[i] = e < P;
+      kk[i] = have[i] ? e / q.tiles : 0;
+      tt[i] = have[i] ? e - kk[i] * q.tiles : 0;
+      idx[i] = base + kk[i] * kstride + tt[i];
+    }
+    while (true) {
+      bool ok = true;
+#pragma unroll
+      for (int i = 0; i < kRecFast; ++i) rec[i] = record_load(rb, idx[i]);
+#pragma unroll
+      for (int i = 0; i < kRecFast; ++i) ok = ok && (!have[i] || record_ready(rec[i], s.epoch));
+      if (ok) break;
+      if (++spins > kMaxSpins) {
+        *s.status = s.epoch;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(2);
+    }
+#pragma unroll
+    for (int i = 0; i < kRecFast; ++i) {
+      if (have[i]) {
+        // copy the lanes out first: __builtin_bit_cast applied directly to a vector element reads element 0
+        const unsigned u0 = rec[i].x, u1 = rec[i].y;
+        body(__builtin_bit_cast(float, u0), __builtin_bit_cast(float, u1), record_count(p, tt[i], k_lo + kk[i], g));
+      }
+    }
+  }
+}
+
+// Every wave waits for the acknowledgement of its device-scope stores; after the workgroup barrier one
+// thread raises the workgroup's flag.
+__device__ __forceinline__ void publish_tile(const SyncArea &s, int64_t idx) {
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    __hip_atomic_store(&s.flags[idx], s.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+// Wait until the `count` flags starting at `first` all carry this call's epoch.
+__device__ __forceinline__ void wait_flags(const SyncArea &s, int64_t first, int count) {
+  int spins = 0;
+  while (true) {
+    int ok = 1;
+    for (int e = threadIdx.x; e < count; e += kBlock)
+      ok &= __hip_atomic_load(&s.flags[first + e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == s.epoch;
+    if (__syncthreads_and(ok)) break;
+    if (++spins > kMaxSpins) {
+      if (threadIdx.x == 0) *s.status = s.epoch;
+      break;
+    }
+    __builtin_amdgcn_s_sleep(2);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Resident forward.  NV = register capacity in rows per lane.  Statistics follow the same definitions
+// as the streaming kernels (count / mean / M2, biased variance, rstd = 1 / sqrt(var + eps);
+// src/gnnhwc/csrc/Welford.h:8-21,66-72, gn_kernel.cu:175,254,291); with the whole tile in registers
+// the per-lane moments are an exact two-pass computation.
+//   records : {mean, M2, epoch} per (n, chunk, group, tile)
+// ---------------------------------------------------------------------------------------------
+template <typename T, typename PT, int VEC, int ACT, int NV>
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 16 ? 4 : 2))) void fused_fwd_kernel(
+    const T *__restrict__ x, T *__restrict__ y, SyncArea sync, const void *w, const void *b, void *mean_out,
+    void *rstd_out, int sdtype, acc_t<T> eps, Plan p) {
+  using A = acc_t<T>;
+  using LV = LaneVec<T, VEC>;
+  __shared__ A sm0[kBlock * VEC];
+  __shared__ A sm1[kBlock * VEC];
+  const PartialGeo q = {p.tiles, p.nchunk, p.lpr * p.vec};
+  const int64_t n = blockIdx.z;
+  const LanePos l = lane_pos(p, n, false);
+  const int rows = l.rows;
+  const int rows_blk = (l.len + p.rpi - 1) / p.rpi;  // most rows any lane of this workgroup owns (<= NV)
+  const int64_t off = (n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC;
+  const int64_t step = (int64_t)p.rpi * p.C;
+  typename LV::raw_t buf[NV];
+  trace_point(sync, 0);
+  if (rows > 0) {
+#pragma unroll
+    for (int u = 0; u < NV; ++u)
+      if (u < rows_blk) buf[u] = LV::load(x + off + (int64_t)clamp_row(u, rows) * step);
+  }
+  A mean[VEC], m2[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) { mean[j] = (A)0; m2[j] = (A)0; }
+  if (rows > 0) {
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      if (u < rows_blk) {
+        const A keep = u < rows ? (A)1 : (A)0;
+        A v[VEC];
+        LV::unpack(buf[u], v);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) mean[j] += keep * v[j];
+      }
+    }
+    const A inv = fast_rcp((A)rows);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) mean[j] *= inv;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      if (u < rows_blk) {
+        const A keep = u < rows ? (A)1 : (A)0;
+        A v[VEC];
+        LV::unpack(buf[u], v);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) { const A d = v[j] - mean[j]; m2[j] += keep * d * d; }
+      }
+    }
+  }
+  const __amdgpu_buffer_rsrc_t rb = record_buffer(sync);
+  trace_point(sync, 1);
+  block_group_moments<A, VEC>(p, l, mean, m2, sm0, sm1, [&](int g, A cnt, A mu, A s2) {
+    (void)cnt;  // the consumers recompute it from the geometry
+    record_store(rb, group_slot(q, p.G, n, l.tile, l.chunk, g), mu, s2, sync.epoch);
+  });
+  trace_point(sync, 2);
+  {
+    // merge the records of the chunk's groups (exact two-pass form, compute_stats_pt2's job:
+    // src/gnnhwc/csrc/gn_kernel.cu:226-292); rstd = 1 / sqrt(M2 / n + eps)
+    const int L = merge_lanes(q, p.D);
+    const int nseg = kBlock / L;
+    const int seg = threadIdx.x / L, sl = threadIdx.x % L;
+    const A total = (A)p.D * (A)p.R;  // elements of a group
+    for (int base = 0; base < l.ng; base += nseg) {
+      const int gi = base + seg;
+      const bool valid = gi < l.ng;
+      const int g = l.g_lo + gi;
+      // each lane folds its records about the mean of its first one ...
+      A nl = (A)0, kl = (A)0, s1 = (A)0, s2 = (A)0;
+      for_group_records(sync, rb, q, p, n, g, valid, L, sl, [&](float mu, float mm, float cnt) {
+        if (nl == (A)0) kl = mu;
+        const A d = mu - kl;
+        nl += cnt;
+        s1 += cnt * d;
+        s2 += mm + cnt * d * d;
+      });
+      const A inv = nl > (A)0 ? (A)1 / nl : (A)0;
+      const A mean_l = kl + s1 * inv;
+      const A m2_l = s2 - s1 * s1 * inv;
+      // ... and the lanes are merged about the first lane's mean
+      const A K = __shfl(mean_l, (int)(threadIdx.x & 63 & ~(L - 1)), 64);
+      const A d = mean_l - K;
+      A t1 = nl * d, t2 = m2_l + nl * d * d;
+      segment_sum2(t1, t2, L);
+      if (valid && sl == 0) {
+        const A dm = t1 / total;
+        const A gmean = K + dm;
+        const A rs = (A)1 / sqrt((t2 - t1 * dm) / total + eps);
+        sm0[gi] = gmean;
+        sm1[gi] = rs;
+        if (l.tile == 0 && g * p.D >= l.cstart) {
+          store_scalar<A>(mean_out, n * p.G + g, sdtype, gmean);
+          store_scalar<A>(rstd_out, n * p.G + g, sdtype, rs);
+        }
+      }
+    }
+    __syncthreads();
+  }
+  trace_point(sync, 3);
+  if (rows > 0) {
+    A sa[VEC], sb[VEC], unused1[VEC], unused2[VEC];
+    lane_coeffs<A, PT, VEC, false>(p, l, w, b, sm0, sm1, nullptr, nullptr, sa, sb, unused1, unused2);
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      if (u < rows_blk) {
+        A v[VEC];
+        LV::unpack(buf[u], v);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] = act_fwd<ACT, A>(v[j] * sa[j] + sb[j]);
+        LV::store(y + off + (int64_t)clamp_row(u, rows) * step, LV::pack(v));
+      }
+    }
+  }
+  trace_point(sync, 4);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Resident backward.  Same algebra as bwd_reduce_kernel + bwd_dx_kernel
+// (src/gnnhwc/csrc/gn_kernel.cu:598-618, 717-727, 783-800, 868-871), with x and dy read once.
+//   partC : [N][tiles][C][2]      records : {A, B, epoch} per (n, chunk, group, tile)
+// ---------------------------------------------------------------------------------------------
+template <typename T, typename PT, int VEC, int ACT, int NV>
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 ? 4 : NV <= 8 ? 3 : NV <= 16 ? 2 : 1))) void fused_bwd_kernel(
+    const T *__restrict__ x, const T *__restrict__ dy, T *__restrict__ dx, const void *mean, const void *rstd, int sdtype,
+    const void *w, const void *b, acc_t<T> *__restrict__ partC, SyncArea sync, void *dw, void *db, Plan p) {
+  using A = acc_t<T>;
+  using LV = LaneVec<T, VEC>;
+  __shared__ A sm1[kBlock * VEC];
+  __shared__ A sm2[kBlock * VEC];
+  __shared__ A sm_mu[kBlock * VEC];
+  __shared__ A sm_rs[kBlock * VEC];
+  const PartialGeo q = {p.tiles, p.nchunk, p.lpr * p.vec};
+  const int64_t n = blockIdx.z;
+  const LanePos l = lane_pos(p, n, false);
+  const __amdgpu_buffer_rsrc_t rb = record_buffer(sync);
+  const int rows = l.rows;
+  const int rows_blk = (l.len + p.rpi - 1) / p.rpi;
+  const int64_t off = (n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC;
+  const int64_t step = (int64_t)p.rpi * p.C;
+  typename LV::raw_t bx[NV], bd[NV];
+  trace_point(sync, 0);
+  if (rows > 0) {
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      if (u < rows_blk) {
+        const int64_t o = off + (int64_t)clamp_row(u, rows) * step;
+        bx[u] = LV::load(x + o);
+        bd[u] = LV::load(dy + o);
+      }
+    }
+  }
+  stage_chunk_stats<A>(mean, rstd, sdtype, p, l, sm_mu, sm_rs);
+  __syncthreads();
+  trace_point(sync, 1);
+  A sa[VEC], sb[VEC], c1[VEC], c2[VEC];
+  {
+    A s1[VEC], s2[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) { s1[j] = (A)0; s2[j] = (A)0; }
+    if (rows > 0) {
+      lane_coeffs<A, PT, VEC, false>(p, l, w, b, sm_mu, sm_rs, nullptr, nullptr, sa, sb, c1, c2);
+#pragma unroll
+      for (int u = 0; u < NV; ++u) {
+        if (u < rows_blk) {
+          const A keep = u < rows ? (A)1 : (A)0;
+          A vx[VEC], vd[VEC];
+          LV::unpack(bx[u], vx);
+          LV::unpack(bd[u], vd);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) {
+            const A g = keep * vd[j] * act_bwd<ACT, A>(vx[j] * sa[j] + sb[j]);
+            s1[j] += g * vx[j];
+            s2[j] += g;
+          }
+        }
+      }
+    }
+    block_channel_sums<A, VEC>(p, l, s1, s2, sm1, sm2);
+  }
+  for (int c = threadIdx.x; c < l.wch; c += kBlock) {
+    const A t1 = sm1[c], t2 = sm2[c];
+    const int64_t idx = ((n * p.tiles + l.tile) * p.C + l.cstart + c) * 2;
+    st_part<true>(partC + idx, t1);
+    st_part<true>(partC + idx + 1, t2);
+    const A gamma = w ? load_param<PT, A>(w, l.cstart + c) : (A)1;
+    sm1[c] = gamma * t1;
+    sm2[c] = gamma * t2;
+  }
+  __syncthreads();
+  {
+    const int L = pow2_ceil_clamped(p.D < l.wch ? p.D : l.wch, 64);
+    const int nseg = kBlock / L;
+    const int seg = threadIdx.x / L, sl = threadIdx.x % L;
+    for (int base = 0; base < l.ng; base += nseg) {
+      const int gi = base + seg;
+      const int g = l.g_lo + gi;
+      const bool valid = gi < l.ng;
+      int ca = 0, cb = 0;
+      if (valid) group_span(p, l, g, ca, cb);
+      A ta = (A)0, tb = (A)0;
+      for (int c = ca + sl; c < cb; c += L) { ta += sm1[c]; tb += sm2[c]; }
+      segment_sum2(ta, tb, L);
+      if (valid && sl == 0) record_store(rb, group_slot(q, p.G, n, l.tile, l.chunk, g), ta, tb, sync.epoch);
+    }
+  }
+  if (dw || db) publish_tile(sync, flag_index(p, n, l.chunk, l.tile));  // partC is complete: for the dgamma / dbeta workgroups
+  else __syncthreads();
+  trace_point(sync, 2);
+  {
+    const int L = merge_lanes(q, p.D);
+    const int nseg = kBlock / L;
+    const int seg = threadIdx.x / L, sl = threadIdx.x % L;
+    for (int base = 0; base < l.ng; base += nseg) {
+      const int gi = base + seg;
+      const bool valid = gi < l.ng;
+      const int g = l.g_lo + gi;
+      A ta = (A)0, tb = (A)0;
+      for_group_records(sync, rb, q, p, n, g, valid, L, sl, [&](float ra, float rbv, float) {
+        ta += ra;
+        tb += rbv;
+      });
+      segment_sum2(ta, tb, L);
+      if (valid && sl == 0) {
+        const A mu = sm_mu[gi];
+        const A rs = sm_rs[gi];
+        const A s = (A)1 / ((A)p.D * (A)p.R);
+        const A k1 = (mu * tb - ta) * s * rs * rs * rs;
+        sm1[gi] = k1;
+        sm2[gi] = -mu * k1 - tb * s * rs;
+      }
+    }
+  }
+  __syncthreads();
+  trace_point(sync, 3);
+  if (rows > 0) {
+    {
+      int gi = (l.cvi * VEC) / p.D;
+      int rem = l.cvi * VEC - gi * p.D;
+      gi -= l.g_lo;
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        c1[j] = sm1[gi];
+        c2[j] = sm2[gi];
+        ++rem;
+        const bool wrap = rem == p.D;
+        rem = wrap ? 0 : rem;
+        gi += wrap ? 1 : 0;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      if (u < rows_blk) {
+        A vx[VEC], vd[VEC];
+        LV::unpack(bx[u], vx);
+        LV::unpack(bd[u], vd);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const A g = vd[j] * act_bwd<ACT, A>(vx[j] * sa[j] + sb[j]);
+          vd[j] = sa[j] * g + (c1[j] * vx[j] + c2[j]);
+        }
+        LV::store(dx + off + (int64_t)clamp_row(u, rows) * step, LV::pack(vd));
+      }
+    }
+  }
+  trace_point(sync, 4);
+  // dgamma / dbeta for the channels of this chunk: row tile 0 of sample 0, once every sample's tiles of
+  // this chunk have published (compute_dweight_dbias, gn_kernel.cu:695-728)
+  if (l.tile == 0 && n == 0 && (dw || db)) {
+    for (int64_t nn = 0; nn < p.N; ++nn) wait_flags(sync, flag_index(p, nn, l.chunk, 0), p.tiles);
+    __syncthreads();
+    const int cw = l.wch < kBlock ? l.wch : kBlock;
+    const int nsl = kBlock / cw;
+    const int cl = threadIdx.x % cw, ts = threadIdx.x / cw;
+    for (int cbase = 0; cbase < l.wch; cbase += cw) {
+      const int c = l.cstart + cbase + cl;
+      A t1 = (A)0, t2 = (A)0;
+      if (cbase + cl < l.wch && ts < nsl) {
+        const int g = c / p.D;
+        for (int64_t nn = 0; nn < p.N; ++nn) {
+          A s1 = (A)0, s2 = (A)0;
+          for (int t = ts; t < p.tiles; t += nsl) {
+            const int64_t idx = ((nn * p.tiles + t) * p.C + c) * 2;
+            s1 += ld_part<true>(partC + idx);
+            s2 += ld_part<true>(partC + idx + 1);
+          }
+          const A mu = load_scalar<A>(mean, nn * p.G + g, sdtype);
+          const A rs = load_scalar<A>(rstd, nn * p.G + g, sdtype);
+          t1 += (s1 - mu * s2) * rs;
+          t2 += s2;
+        }
+      }
+      __syncthreads();
+      if (ts < nsl) { sm1[ts * cw + cl] = t1; sm2[ts * cw + cl] = t2; }
+      __syncthreads();
+      if (ts == 0 && cbase + cl < l.wch) {
+        A r1 = (A)0, r2 = (A)0;
+        for (int s = 0; s < nsl; ++s) { r1 += sm1[s * cw + cl]; r2 += sm2[s * cw + cl]; }
+        if (dw) store_param<PT, A>(dw, c, r1);
+        if (db) store_param<PT, A>(db, c, r2);
+      }
+    }
+    trace_point(sync, 5);
+  }
+}
+
+}  // namespace gn

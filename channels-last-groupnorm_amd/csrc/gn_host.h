@@ -62,6 +62,21 @@ inline BwdWorkspace bwd_workspace(const Plan &p) {
   w.total = w.compactG + align_up((size_t)p.N * p.G * 2, 64);
   return w;
 }
+// The resident kernels keep their partial results and one flag per workgroup in the same workspace.
+constexpr int kMaxResidentBlocks = 4 * kNumCU;
+inline size_t resident_rec_bytes(int64_t G) { return (size_t)16 * G * kMaxResidentBlocks; }
+inline size_t resident_fwd_bytes(int64_t G) { return align_up(resident_rec_bytes(G), 256) + 256; }
+// chunk_channels = channels per workgroup (lpr * vec): N * tiles * C = workgroups * chunk_channels
+inline size_t resident_bwd_bytes(int64_t chunk_channels, int64_t G) {
+  return align_up((size_t)2 * chunk_channels * kMaxResidentBlocks * 4, 256) + align_up(resident_rec_bytes(G), 256) +
+         (size_t)kMaxResidentBlocks * 8 + 256;
+}
+// A fresh nonzero 64-bit value per call (gn_api.hip).
+unsigned long long next_epoch();
+bool resident_enabled();
+// Device buffer for in-kernel timestamps when GNNHWC_TRACE=1, else null.
+unsigned long long *trace_buffer();
+
 // Consumers merge the tile partials of their own groups unless that would be more than
 // kMaxInlineEntries entries per workgroup; then a compaction kernel runs in between.
 inline bool needs_compaction(const Plan &p) {

@@ -1,6 +1,7 @@
 // Kernel instantiations and launch sequences for ONE element type, selected with -DGN_INST_DTYPE=0..3
 // (f32, f64, f16, bf16).  Built four times so the four types compile in parallel.
 #include "gn_host.h"
+#include "gn_fused.h"
 #include "gn_kernels.h"
 
 #ifndef GN_INST_DTYPE
@@ -54,7 +55,143 @@ template <typename PT, int VEC> void launch_apply_act(const FwdArgs &a, const A 
   }
 }
 
+// ---- resident (single-launch) path ----------------------------------------------------------------
+// Workgroups that can be resident at once for a kernel: occupancy reported by the runtime times the CUs.
+template <typename K> int resident_slots(K kernel) {
+  int per_cu = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kBlock, 0) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  const int slots = per_cu * cus;
+  return slots < kMaxResidentBlocks ? slots : kMaxResidentBlocks;
+}
+
+// Choose the row tiling of a resident launch: rows per lane <= nv, all workgroups resident, and the
+// workgroups spread as evenly over the CUs as the shape allows.  Returns false if it does not fit.
+bool resident_tiling(const Plan &base, int nv, int slots, Plan &out) {
+  const int64_t columns = base.N * base.nchunk;
+  if (slots <= 0 || columns > slots || base.N > 65535) return false;
+  const int64_t tiles_min = (base.R + (int64_t)nv * base.rpi - 1) / ((int64_t)nv * base.rpi);
+  const int64_t tiles_max = slots / columns;
+  if (tiles_min > tiles_max) return false;
+  int64_t best = -1;
+  double best_eff = -1.0;
+  for (int64_t t = tiles_min; t <= tiles_max; ++t) {
+    int64_t rows = (base.R + t - 1) / t;
+    rows = (rows + base.rpi - 1) / base.rpi * base.rpi;
+    if ((base.R + rows - 1) / rows != t) continue;  // this tile count cannot be realised with equal tiles
+    const int64_t blocks = columns * t;
+    const double eff = (double)blocks / (double)((blocks + kNumCU - 1) / kNumCU * kNumCU);
+    if (eff > best_eff + 1e-9) { best_eff = eff; best = t; }
+  }
+  if (best < 0) return false;
+  out = base;
+  int64_t rows = (base.R + best - 1) / best;
+  rows = (rows + base.rpi - 1) / base.rpi * base.rpi;
+  out.tile_rows = (int)rows;
+  out.tiles = (int)best;
+  out.nblocks = columns * best;
+  return true;
+}
+
+struct ResidentWorkspace {
+  A *partC;  // backward only
+  SyncArea sync;
+};
+ResidentWorkspace resident_fwd_ws(void *ws, const Plan &p) {
+  ResidentWorkspace r;
+  char *base = (char *)ws;
+  r.partC = nullptr;
+  r.sync.recs = base;
+  r.sync.rec_bytes = (unsigned)resident_rec_bytes(p.G);
+  r.sync.flags = nullptr;
+  r.sync.status = (unsigned long long *)(base + align_up(resident_rec_bytes(p.G), 256));
+  r.sync.epoch = next_epoch();
+  r.sync.trace = trace_buffer();
+  return r;
+}
+ResidentWorkspace resident_bwd_ws(void *ws, const Plan &p) {
+  ResidentWorkspace r;
+  char *base = (char *)ws;
+  const size_t cc = (size_t)p.lpr * p.vec;
+  r.partC = (A *)base;
+  char *recs = base + align_up((size_t)2 * cc * kMaxResidentBlocks * 4, 256);
+  r.sync.recs = recs;
+  r.sync.rec_bytes = (unsigned)resident_rec_bytes(p.G);
+  char *f = recs + align_up(resident_rec_bytes(p.G), 256);
+  r.sync.flags = (unsigned long long *)f;
+  r.sync.status = (unsigned long long *)(f + (size_t)kMaxResidentBlocks * 8);
+  r.sync.epoch = next_epoch();
+  r.sync.trace = trace_buffer();
+  return r;
+}
+
+template <typename PT, int ACT, int NV> bool try_resident_fwd_nv(const FwdArgs &a) {
+  auto kernel = fused_fwd_kernel<elem_t, PT, kVec, ACT, NV>;
+  static const int slots = resident_slots(kernel);
+  Plan p;
+  if (!resident_tiling(a.plan, NV, slots, p)) return false;
+  const ResidentWorkspace r = resident_fwd_ws(a.ws, p);
+  ProfileScope s(kKindFusedFwd, a.stream);
+  hipLaunchKernelGGL(kernel, tile_grid(p, 0), dim3(kBlock), 0, a.stream, (const elem_t *)a.x, (elem_t *)a.y, r.sync, a.w, a.b,
+                     a.mean, a.rstd, a.sdtype, (A)a.eps, p);
+  return true;
+}
+template <typename PT, int ACT> bool try_resident_fwd_act(const FwdArgs &a) {
+  return try_resident_fwd_nv<PT, ACT, 4>(a) || try_resident_fwd_nv<PT, ACT, 8>(a) || try_resident_fwd_nv<PT, ACT, 16>(a) ||
+         try_resident_fwd_nv<PT, ACT, 32>(a);
+}
+template <typename PT> bool try_resident_fwd_pt(const FwdArgs &a) {
+  switch (a.act) {
+    case GN_ACT_IDENTITY: return try_resident_fwd_act<PT, GN_ACT_IDENTITY>(a);
+    case GN_ACT_RELU: return try_resident_fwd_act<PT, GN_ACT_RELU>(a);
+    case GN_ACT_SILU: return try_resident_fwd_act<PT, GN_ACT_SILU>(a);
+    case GN_ACT_GELU: return try_resident_fwd_act<PT, GN_ACT_GELU>(a);
+    default: return try_resident_fwd_act<PT, GN_ACT_GELU_TANH>(a);
+  }
+}
+bool try_resident_fwd(const FwdArgs &a) {
+  if (!resident_enabled() || a.plan.vec == 1 || sizeof(A) != 4) return false;
+  return a.pdtype == GN_INST_DTYPE ? try_resident_fwd_pt<elem_t>(a) : try_resident_fwd_pt<wide_param_t>(a);
+}
+
+template <typename PT, int ACT, int NV> bool try_resident_bwd_nv(const BwdArgs &a) {
+  auto kernel = fused_bwd_kernel<elem_t, PT, kVec, ACT, NV>;
+  static const int slots = resident_slots(kernel);
+  Plan p;
+  if (!resident_tiling(a.plan, NV, slots, p)) return false;
+  const ResidentWorkspace r = resident_bwd_ws(a.ws, p);
+  ProfileScope s(kKindFusedBwd, a.stream);
+  hipLaunchKernelGGL(kernel, tile_grid(p, 0), dim3(kBlock), 0, a.stream, (const elem_t *)a.x, (const elem_t *)a.dy,
+                     (elem_t *)a.dx, a.mean, a.rstd, a.sdtype, a.w, a.b, r.partC, r.sync, a.dw, a.db, p);
+  return true;
+}
+template <typename PT, int ACT> bool try_resident_bwd_act(const BwdArgs &a) {
+  return try_resident_bwd_nv<PT, ACT, 4>(a) || try_resident_bwd_nv<PT, ACT, 8>(a) || try_resident_bwd_nv<PT, ACT, 16>(a) ||
+         try_resident_bwd_nv<PT, ACT, 32>(a);
+}
+template <typename PT> bool try_resident_bwd_pt(const BwdArgs &a) {
+  switch (a.act) {
+    case GN_ACT_IDENTITY: return try_resident_bwd_act<PT, GN_ACT_IDENTITY>(a);
+    case GN_ACT_RELU: return try_resident_bwd_act<PT, GN_ACT_RELU>(a);
+    case GN_ACT_SILU: return try_resident_bwd_act<PT, GN_ACT_SILU>(a);
+    case GN_ACT_GELU: return try_resident_bwd_act<PT, GN_ACT_GELU>(a);
+    default: return try_resident_bwd_act<PT, GN_ACT_GELU_TANH>(a);
+  }
+}
+bool try_resident_bwd(const BwdArgs &a) {
+  if (!resident_enabled() || a.plan.vec == 1 || sizeof(A) != 4) return false;
+  return a.pdtype == GN_INST_DTYPE ? try_resident_bwd_pt<elem_t>(a) : try_resident_bwd_pt<wide_param_t>(a);
+}
+
 template <int VEC> hipError_t fwd_impl(const FwdArgs &a) {
+  if (VEC != 1 && try_resident_fwd(a)) return hipGetLastError();
   const Plan &p = a.plan;
   const FwdWorkspace ws = fwd_workspace(p);
   A *base = (A *)a.ws;
@@ -120,6 +257,7 @@ template <typename PT, int VEC> void bwd_act(const BwdArgs &a) {
   }
 }
 template <int VEC> hipError_t bwd_impl(const BwdArgs &a) {
+  if (VEC != 1 && try_resident_bwd(a)) return hipGetLastError();
   if (a.pdtype == GN_INST_DTYPE) bwd_act<elem_t, VEC>(a);
   else bwd_act<wide_param_t, VEC>(a);
   return hipGetLastError();

@@ -86,6 +86,19 @@ __device__ __forceinline__ void double_buffered(int nb, ISSUE &&issue, CONSUME &
 }
 __device__ __forceinline__ int clamp_row(int idx, int rows) { return idx < rows ? idx : rows - 1; }
 
+// Partial results are ordinary cached data between two launches, but inside a resident launch they are
+// exchanged between workgroups on different XCDs, whose L2 caches are not coherent with each other.
+// COH selects device-scope accesses (write-through stores, cache-bypassing loads), which makes the
+// exchange work without any L2 write-back / invalidate fence.
+template <bool COH, typename A> __device__ __forceinline__ A ld_part(const A *p) {
+  if constexpr (COH) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  else return *p;
+}
+template <bool COH, typename A> __device__ __forceinline__ void st_part(A *p, A v) {
+  if constexpr (COH) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  else *p = v;
+}
+
 template <typename PT, typename A> __device__ __forceinline__ A load_param(const void *p, int64_t i) {
   A v[1];
   LaneVec<PT, 1>::unpack(LaneVec<PT, 1>::load((const PT *)p + i), v);
@@ -194,58 +207,152 @@ __device__ __forceinline__ void lane_stats(const T *__restrict__ x, const Plan &
   double_buffered(nb, issue, consume);
 }
 
+// Rows of the tile owned by the lane rows of wavefront wv (64 / lpr lane rows per wavefront).
+__device__ __forceinline__ int wave_rows(const Plan &p, const LanePos &l, int wv) {
+  const int tpw = 64 / p.lpr;
+  int extra = l.rows_rem - wv * tpw;
+  extra = extra < 0 ? 0 : (extra > tpw ? tpw : extra);
+  return tpw * l.rows_base + extra;
+}
+
 // Merge the per-lane moments of a workgroup into one (count, mean, M2) triple per group of the chunk and
-// hand each to emit(g, count, mean, M2) (called by one lane per group).  Uses the exact two-pass form,
-// first across the lane rows of a channel, then across the channels of a group.
+// hand each to emit(g, count, mean, M2) (called by one lane per group).
+// When the lanes of a row divide the wavefront (lpr | 64, the usual case) the lane rows of a wavefront are
+// first merged with butterfly shuffles (Chan's update, Welford.h:44-65), so LDS only carries one entry per
+// wavefront and channel; otherwise every lane row goes through LDS.  The entries of a group are then
+// merged with the exact two-pass form.
 template <typename A, int VEC, typename EMIT>
 __device__ __forceinline__ void block_group_moments(const Plan &p, const LanePos &l, const A (&mean)[VEC],
                                                     const A (&m2)[VEC], A *sm_mean, A *sm_m2, EMIT &&emit) {
   const int W = p.lpr * VEC;
-  if (l.active) {
+  const bool wave_path = (64 % p.lpr) == 0;
+  int nrow;  // LDS rows per channel after the first step
+  if (wave_path) {
+    A mw[VEC], qw[VEC];
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-      sm_mean[l.ty * W + l.tx * VEC + j] = mean[j];
-      sm_m2[l.ty * W + l.tx * VEC + j] = m2[j];
+    for (int j = 0; j < VEC; ++j) { mw[j] = mean[j]; qw[j] = m2[j]; }
+    A cnt = (A)l.rows;
+    for (int off = p.lpr; off < 64; off <<= 1) {
+      const A ocnt = shfl_xor_acc(cnt, off, 64);
+      const A nn = cnt + ocnt;
+      const A f = nn > (A)0 ? ocnt * fast_rcp(nn) : (A)0;
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const A om = shfl_xor_acc(mw[j], off, 64);
+        const A oq = shfl_xor_acc(qw[j], off, 64);
+        const A d = om - mw[j];
+        mw[j] += d * f;
+        qw[j] += oq + d * d * cnt * f;
+      }
+      cnt = nn;
     }
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    if (lane < p.lpr && l.cvi < p.cv) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        sm_mean[wv * W + lane * VEC + j] = mw[j];
+        sm_m2[wv * W + lane * VEC + j] = qw[j];
+      }
+    }
+    nrow = kBlock / 64;
+  } else {
+    if (l.active) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        sm_mean[l.ty * W + l.tx * VEC + j] = mean[j];
+        sm_m2[l.ty * W + l.tx * VEC + j] = m2[j];
+      }
+    }
+    nrow = l.len < p.rpi ? l.len : p.rpi;
   }
   __syncthreads();
-  const int rows_used = l.len < p.rpi ? l.len : p.rpi;
-  for (int c = threadIdx.x; c < l.wch; c += kBlock) {
-    A sm = (A)0;
-    for (int ty = 0; ty < rows_used; ++ty) sm += (A)(l.rows_base + (ty < l.rows_rem ? 1 : 0)) * sm_mean[ty * W + c];
-    const A mu = sm / (A)l.len;
-    A s2 = (A)0;
-    for (int ty = 0; ty < rows_used; ++ty) {
-      const A d = sm_mean[ty * W + c] - mu;
-      s2 += sm_m2[ty * W + c] + (A)(l.rows_base + (ty < l.rows_rem ? 1 : 0)) * d * d;
-    }
-    sm_mean[c] = mu;  // the column's result replaces its row 0 (only this thread touches the column)
-    sm_m2[c] = s2;
-  }
-  __syncthreads();
-  const int L = pow2_ceil_clamped(p.D < l.wch ? p.D : l.wch, 64);
+  const int nc_max = p.D < l.wch ? p.D : l.wch;
+  const int L = pow2_ceil_clamped(nc_max, 16);  // lanes per group: a DPP row at most
   const int nseg = kBlock / L;
   const int seg = threadIdx.x / L, sl = threadIdx.x % L;
+  const int tpw = wave_path ? 64 / p.lpr : 1;
   for (int base = 0; base < l.ng; base += nseg) {
     const int gi = base + seg;
     const int g = l.g_lo + gi;
     const bool valid = gi < l.ng;
     int ca = 0, cb = 0;
     if (valid) group_span(p, l, g, ca, cb);
-    A sm = (A)0;
-    for (int c = ca + sl; c < cb; c += L) sm += sm_mean[c];
-    sm = segment_sum(sm, L);
-    const A nch = (A)(cb - ca);
-    const A mu = valid ? sm / nch : (A)0;
-    A s2 = (A)0;
-    for (int c = ca + sl; c < cb; c += L) {
-      const A d = sm_mean[c] - mu;
-      s2 += sm_m2[c] + (A)l.len * d * d;
+    // one pass about the pivot K = mean of the group's first entry
+    const A K = valid ? sm_mean[ca] : (A)0;
+    A s1 = (A)0, s2 = (A)0;
+    for (int c = ca + sl; c < cb; c += L)
+      for (int r = 0; r < nrow; ++r) {
+        int rows_r;
+        if (wave_path) {
+          int extra = l.rows_rem - r * tpw;
+          extra = extra < 0 ? 0 : (extra > tpw ? tpw : extra);
+          rows_r = tpw * l.rows_base + extra;
+        } else {
+          rows_r = l.rows_base + (r < l.rows_rem ? 1 : 0);
+        }
+        const A rc = (A)rows_r;
+        const A d = sm_mean[r * W + c] - K;
+        s1 += rc * d;
+        s2 += sm_m2[r * W + c] + rc * d * d;
+      }
+    segment_sum2(s1, s2, L);
+    if (valid && sl == 0) {
+      const A total = (A)(cb - ca) * (A)l.len;
+      const A dm = s1 / total;
+      emit(g, total, K + dm, s2 - s1 * dm);
     }
-    s2 = segment_sum(s2, L);
-    if (valid && sl == 0) emit(g, nch * (A)l.len, mu, s2);
   }
   __syncthreads();  // the LDS arrays may be reused by the caller
+}
+
+// Sum the per-lane (s1, s2) pairs of a workgroup over its lane rows: afterwards sm1[c], sm2[c] hold the
+// tile's sums for channel c of the chunk (c < wch).  Same two routes as block_group_moments.
+template <typename A, int VEC>
+__device__ __forceinline__ void block_channel_sums(const Plan &p, const LanePos &l, const A (&s1)[VEC], const A (&s2)[VEC],
+                                                   A *sm1, A *sm2) {
+  const int W = p.lpr * VEC;
+  int nrow;
+  if ((64 % p.lpr) == 0) {
+    A a1[VEC], a2[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) { a1[j] = s1[j]; a2[j] = s2[j]; }
+    for (int off = p.lpr; off < 64; off <<= 1) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        a1[j] += shfl_xor_acc(a1[j], off, 64);
+        a2[j] += shfl_xor_acc(a2[j], off, 64);
+      }
+    }
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    if (lane < p.lpr && l.cvi < p.cv) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        sm1[wv * W + lane * VEC + j] = a1[j];
+        sm2[wv * W + lane * VEC + j] = a2[j];
+      }
+    }
+    nrow = kBlock / 64;
+  } else {
+    if (l.active) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        sm1[l.ty * W + l.tx * VEC + j] = s1[j];
+        sm2[l.ty * W + l.tx * VEC + j] = s2[j];
+      }
+    }
+    nrow = p.rpi;
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < l.wch; c += kBlock) {
+    A t1 = (A)0, t2 = (A)0;
+    for (int r = 0; r < nrow; ++r) {
+      t1 += sm1[r * W + c];
+      t2 += sm2[r * W + c];
+    }
+    sm1[c] = t1;  // replaces row 0 of the column (only this thread touches the column)
+    sm2[c] = t2;
+  }
+  __syncthreads();
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -276,7 +383,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) voi
 
 // Merge the P = tiles * (chunks holding a piece of g) partial triples of group g with `L` lanes; every
 // lane of the segment returns the merged triple (exact two-pass form).
-template <typename A>
+template <typename A, bool COH>
 __device__ __forceinline__ Moments<A> merge_group_partials(const A *__restrict__ part, int64_t plane, const PartialGeo &q,
                                                            int G, int D, int64_t n, int g, bool valid, int L, int sl) {
   int k_lo = 0, nk = 1;
@@ -289,9 +396,9 @@ __device__ __forceinline__ Moments<A> merge_group_partials(const A *__restrict__
   for (int e = sl; e < P; e += L) {
     const int k = e / q.tiles, t = e - k * q.tiles;
     const int64_t slot = base + k * kstride + t;
-    const A cn = part[slot];
+    const A cn = ld_part<COH>(part + slot);
     sn += cn;
-    sm += cn * part[plane + slot];
+    sm += cn * ld_part<COH>(part + plane + slot);
   }
   sn = segment_sum(sn, L);
   sm = segment_sum(sm, L);
@@ -302,8 +409,8 @@ __device__ __forceinline__ Moments<A> merge_group_partials(const A *__restrict__
   for (int e = sl; e < P; e += L) {
     const int k = e / q.tiles, t = e - k * q.tiles;
     const int64_t slot = base + k * kstride + t;
-    const A d = part[plane + slot] - r.mean;
-    s2 += part[2 * plane + slot] + part[slot] * d * d;
+    const A d = ld_part<COH>(part + plane + slot) - r.mean;
+    s2 += ld_part<COH>(part + 2 * plane + slot) + ld_part<COH>(part + slot) * d * d;
   }
   r.m2 = segment_sum(s2, L);
   return r;
@@ -322,7 +429,7 @@ __global__ __launch_bounds__(kBlock) void stats_compact_kernel(const A *__restri
   const bool valid = item < p.N * p.G;
   const int64_t n = valid ? item / p.G : 0;
   const int g = valid ? (int)(item - n * p.G) : 0;
-  const Moments<A> m = merge_group_partials<A>(part, group_plane(q, p.G, p.N), q, p.G, p.D, n, g, valid, 64, lane);
+  const Moments<A> m = merge_group_partials<A, false>(part, group_plane(q, p.G, p.N), q, p.G, p.D, n, g, valid, 64, lane);
   if (valid && lane == 0) {
     const int64_t oplane = p.N * p.G;
     out[item] = m.n;
@@ -334,7 +441,7 @@ __global__ __launch_bounds__(kBlock) void stats_compact_kernel(const A *__restri
 // Consumer prologue of the forward: merge the tile partials of the chunk's groups into mean / rstd
 // (compute_stats_pt2, src/gnnhwc/csrc/gn_kernel.cu:226-292: rstd = 1 / sqrt(M2 / n + eps)), leave them in
 // LDS indexed by (g - g_lo), and let the workgroups of row tile 0 report them to the caller's outputs.
-template <typename A>
+template <typename A, bool COH>
 __device__ __forceinline__ void merge_chunk_stats(const A *__restrict__ part, const PartialGeo &q, const Plan &p,
                                                   const LanePos &l, A eps, A *sm_mu, A *sm_rs, void *mean_out,
                                                   void *rstd_out, int sdtype) {
@@ -346,7 +453,7 @@ __device__ __forceinline__ void merge_chunk_stats(const A *__restrict__ part, co
     const int gi = base + seg;
     const bool valid = gi < l.ng;
     const int g = l.g_lo + gi;
-    const Moments<A> m = merge_group_partials<A>(part, plane, q, p.G, p.D, l.n, g, valid, L, sl);
+    const Moments<A> m = merge_group_partials<A, COH>(part, plane, q, p.G, p.D, l.n, g, valid, L, sl);
     if (valid && sl == 0) {
       const A rs = (A)1 / sqrt(m.m2 / m.n + eps);
       sm_mu[gi] = m.mean;
@@ -452,7 +559,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) voi
       }
     };
     if (nb > 0) issue(std::integral_constant<int, 0>{}, 0);  // in flight while the statistics are merged
-    merge_chunk_stats<A>(part, q, p, l, eps, sm_mu, sm_rs, mean_out, rstd_out, sdtype);
+    merge_chunk_stats<A, false>(part, q, p, l, eps, sm_mu, sm_rs, mean_out, rstd_out, sdtype);
     if (nb > 0) {
       lane_coeffs<A, PT, VEC, false>(p, l, w, b, sm_mu, sm_rs, nullptr, nullptr, sa, sb, unused1, unused2);
       double_buffered(nb, issue, consume);
@@ -483,7 +590,6 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) voi
   const int64_t plane = group_plane(q, p.G, p.N);
   for (int64_t n = blockIdx.z; n < p.N; n += gridDim.z) {
     const LanePos l = lane_pos(p, n, false);
-    const int W = p.lpr * VEC;
     const int rows = l.rows;
     const int nb = (rows + U - 1) / U;
     const int64_t off = (n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC;
@@ -516,27 +622,16 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) voi
     if (nb > 0) issue(std::integral_constant<int, 0>{}, 0);
     stage_chunk_stats<A>(mean, rstd, sdtype, p, l, sm_mu, sm_rs);
     __syncthreads();
-    if (l.active) {
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) { s1[j] = (A)0; s2[j] = (A)0; }
-      if (nb > 0) {
-        lane_coeffs<A, PT, VEC, false>(p, l, w, b, sm_mu, sm_rs, nullptr, nullptr, sa, sb, unused1, unused2);
-        double_buffered(nb, issue, consume);
-      }
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        sm1[l.ty * W + l.tx * VEC + j] = s1[j];
-        sm2[l.ty * W + l.tx * VEC + j] = s2[j];
-      }
+    for (int j = 0; j < VEC; ++j) { s1[j] = (A)0; s2[j] = (A)0; }
+    if (nb > 0) {
+      lane_coeffs<A, PT, VEC, false>(p, l, w, b, sm_mu, sm_rs, nullptr, nullptr, sa, sb, unused1, unused2);
+      double_buffered(nb, issue, consume);
     }
-    __syncthreads();
-    // per channel: sum the lane rows; keep gamma-weighted copies in row 0 for the group sums
+    block_channel_sums<A, VEC>(p, l, s1, s2, sm1, sm2);
+    // per channel: publish the tile sums; keep gamma-weighted copies for the group sums
     for (int c = threadIdx.x; c < l.wch; c += kBlock) {
-      A t1 = (A)0, t2 = (A)0;
-      for (int ty = 0; ty < p.rpi; ++ty) {
-        t1 += sm1[ty * W + c];
-        t2 += sm2[ty * W + c];
-      }
+      const A t1 = sm1[c], t2 = sm2[c];
       const int64_t idx = ((n * p.tiles + l.tile) * p.C + l.cstart + c) * 2;
       partC[idx] = t1;
       partC[idx + 1] = t2;
@@ -571,7 +666,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) voi
 }
 
 // Sum the tile partials (A, B) of group g with L lanes; every lane of the segment gets the sums.
-template <typename A>
+template <typename A, bool COH>
 __device__ __forceinline__ void sum_group_partials(const A *__restrict__ partG, int64_t plane, const PartialGeo &q, int G,
                                                    int D, int64_t n, int g, bool valid, int L, int sl, A &ta, A &tb) {
   int k_lo = 0, nk = 1;
@@ -584,8 +679,8 @@ __device__ __forceinline__ void sum_group_partials(const A *__restrict__ partG, 
   for (int e = sl; e < P; e += L) {
     const int k = e / q.tiles, t = e - k * q.tiles;
     const int64_t slot = base + k * kstride + t;
-    ta += partG[slot];
-    tb += partG[plane + slot];
+    ta += ld_part<COH>(partG + slot);
+    tb += ld_part<COH>(partG + plane + slot);
   }
   ta = segment_sum(ta, L);
   tb = segment_sum(tb, L);
@@ -607,7 +702,7 @@ __global__ __launch_bounds__(kBlock) void bwd_compact_kernel(const A *__restrict
     const int64_t n = valid ? item / p.G : 0;
     const int g = valid ? (int)(item - n * p.G) : 0;
     A ta, tb;
-    sum_group_partials<A>(partG, group_plane(q, p.G, p.N), q, p.G, p.D, n, g, valid, 64, lane, ta, tb);
+    sum_group_partials<A, false>(partG, group_plane(q, p.G, p.N), q, p.G, p.D, n, g, valid, 64, lane, ta, tb);
     if (valid && lane == 0) {
       outG[item] = ta;
       outG[p.N * p.G + item] = tb;
@@ -738,7 +833,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) voi
         const bool valid = gi < l.ng;
         const int g = l.g_lo + gi;
         A ta, tb;
-        sum_group_partials<A>(partG, plane, q, p.G, p.D, n, g, valid, L, sl, ta, tb);
+        sum_group_partials<A, false>(partG, plane, q, p.G, p.D, n, g, valid, L, sl, ta, tb);
         if (valid && sl == 0) {
           const A mu = load_scalar<A>(mean, n * p.G + g, sdtype);
           const A rs = load_scalar<A>(rstd, n * p.G + g, sdtype);

@@ -118,6 +118,15 @@ int gnnhwc_profile_collect(int64_t *launches /* [GNNHWC_NUM_KERNEL_KINDS] */,
                            double *total_ms /* [GNNHWC_NUM_KERNEL_KINDS] */);
 const char *gnnhwc_kernel_kind_name(int kind);
 
+/*
+ * In-kernel timeline of the single-launch kernels, for tuning (no counterpart in the reference; its
+ * nearest relative is the DEBUG(...) launch-parameter printf, gn_kernel.cu:13-19).  With GNNHWC_TRACE=1
+ * in the environment at the first call, thread 0 of every workgroup of a single-launch kernel writes a
+ * 100 MHz wall-clock stamp at up to 8 phase boundaries.  This call synchronises the device and copies
+ * `count` 64-bit words, laid out [workgroup][8], from the most recent such launch.
+ */
+int gnnhwc_debug_read_trace(unsigned long long *out, int64_t count);
+
 #ifdef __cplusplus
 }
 #endif
