@@ -224,9 +224,11 @@ unsigned long long *trace_buffer() {
   }();
   return buf;
 }
+std::atomic<int> g_resident{-1};  // -1: follow the environment
 bool resident_enabled() {
   static const int off = env_int("GNNHWC_DISABLE_RESIDENT", 0);
-  return off == 0;
+  const int v = g_resident.load(std::memory_order_relaxed);
+  return v < 0 ? off == 0 : v != 0;
 }
 
 void profile_before(int kind, hipStream_t stream) {
@@ -368,6 +370,12 @@ int gnnhwc_profile_collect(int64_t *launches, double *total_ms) {
   }
   g_timed.clear();
   return rc;
+}
+
+int gnnhwc_set_resident(int on) {
+  const int before = resident_enabled() ? 1 : 0;
+  g_resident.store(on ? 1 : 0, std::memory_order_relaxed);
+  return before;
 }
 
 int gnnhwc_debug_read_trace(unsigned long long *out, int64_t count) {

@@ -38,6 +38,7 @@ struct SyncArea {
   unsigned rec_bytes;
   unsigned long long *flags;  // [N][nchunk][tiles]
   unsigned long long epoch;   // value that marks "written in this call"
+  const unsigned long long *generation;  // optional device word folded into the epoch (see resident_epoch)
   unsigned long long *status; // set to the epoch if a wait of this call timed out
   unsigned long long *trace;  // optional [workgroup][kTracePoints] timestamps (100 MHz wall clock), else null
 };
@@ -48,6 +49,16 @@ __device__ __forceinline__ void trace_point(const SyncArea &s, int point) {
     const int64_t b = ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
     if (b < kMaxResidentBlocksDev) s.trace[b * kTracePoints + point] = wall_clock64();
   }
+}
+
+// A launch recorded into a HIP graph is replayed with identical kernel arguments, so the host cannot give
+// each replay a fresh epoch.  For captured launches the host therefore records a one-thread kernel in front
+// that increments a generation word in the workspace, and the epoch becomes host value + generation * odd.
+template <int UNUSED> __global__ void bump_generation_kernel(unsigned long long *generation) { *generation += 1; }
+__device__ __forceinline__ SyncArea resident_epoch(SyncArea s) {
+  if (s.generation) s.epoch += *s.generation * 0x9E3779B97F4A7C15ull;
+  if (s.epoch == 0) s.epoch = 1;
+  return s;
 }
 
 __device__ __forceinline__ int64_t flag_index(const Plan &p, int64_t n, int k, int t) {
@@ -168,10 +179,11 @@ __device__ __forceinline__ void wait_flags(const SyncArea &s, int64_t first, int
 // ---------------------------------------------------------------------------------------------
 template <typename T, typename PT, int VEC, int ACT, int NV>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 16 ? 4 : 2))) void fused_fwd_kernel(
-    const T *__restrict__ x, T *__restrict__ y, SyncArea sync, const void *w, const void *b, void *mean_out,
+    const T *__restrict__ x, T *__restrict__ y, SyncArea sync_arg, const void *w, const void *b, void *mean_out,
     void *rstd_out, int sdtype, acc_t<T> eps, Plan p) {
   using A = acc_t<T>;
   using LV = LaneVec<T, VEC>;
+  const SyncArea sync = resident_epoch(sync_arg);
   __shared__ A sm0[kBlock * VEC];
   __shared__ A sm1[kBlock * VEC];
   const PartialGeo q = {p.tiles, p.nchunk, p.lpr * p.vec};
@@ -291,9 +303,10 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 16
 template <typename T, typename PT, int VEC, int ACT, int NV>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 ? 4 : NV <= 8 ? 3 : NV <= 16 ? 2 : 1))) void fused_bwd_kernel(
     const T *__restrict__ x, const T *__restrict__ dy, T *__restrict__ dx, const void *mean, const void *rstd, int sdtype,
-    const void *w, const void *b, acc_t<T> *__restrict__ partC, SyncArea sync, void *dw, void *db, Plan p) {
+    const void *w, const void *b, acc_t<T> *__restrict__ partC, SyncArea sync_arg, void *dw, void *db, Plan p) {
   using A = acc_t<T>;
   using LV = LaneVec<T, VEC>;
+  const SyncArea sync = resident_epoch(sync_arg);
   __shared__ A sm1[kBlock * VEC];
   __shared__ A sm2[kBlock * VEC];
   __shared__ A sm_mu[kBlock * VEC];

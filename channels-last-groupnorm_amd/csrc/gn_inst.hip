@@ -103,7 +103,25 @@ bool resident_tiling(const Plan &base, int nv, int slots, Plan &out) {
 struct ResidentWorkspace {
   A *partC;  // backward only
   SyncArea sync;
+  unsigned long long *generation;  // device word behind the status word
 };
+// True while `stream` is recording into a HIP graph.
+bool stream_is_capturing(hipStream_t stream) {
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &st) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return st != hipStreamCaptureStatusNone;
+}
+// Captured launches get their per-replay epoch from a generation word bumped by a kernel recorded in front.
+void arm_generation(ResidentWorkspace &r, hipStream_t stream) {
+  r.sync.generation = nullptr;
+  if (stream_is_capturing(stream)) {
+    hipLaunchKernelGGL(bump_generation_kernel<GN_INST_DTYPE>, dim3(1), dim3(1), 0, stream, r.generation);
+    r.sync.generation = r.generation;
+  }
+}
 ResidentWorkspace resident_fwd_ws(void *ws, const Plan &p) {
   ResidentWorkspace r;
   char *base = (char *)ws;
@@ -112,6 +130,7 @@ ResidentWorkspace resident_fwd_ws(void *ws, const Plan &p) {
   r.sync.rec_bytes = (unsigned)resident_rec_bytes(p.G);
   r.sync.flags = nullptr;
   r.sync.status = (unsigned long long *)(base + align_up(resident_rec_bytes(p.G), 256));
+  r.generation = r.sync.status + 1;
   r.sync.epoch = next_epoch();
   r.sync.trace = trace_buffer();
   return r;
@@ -127,6 +146,7 @@ ResidentWorkspace resident_bwd_ws(void *ws, const Plan &p) {
   char *f = recs + align_up(resident_rec_bytes(p.G), 256);
   r.sync.flags = (unsigned long long *)f;
   r.sync.status = (unsigned long long *)(f + (size_t)kMaxResidentBlocks * 8);
+  r.generation = r.sync.status + 1;
   r.sync.epoch = next_epoch();
   r.sync.trace = trace_buffer();
   return r;
@@ -137,7 +157,8 @@ template <typename PT, int ACT, int NV> bool try_resident_fwd_nv(const FwdArgs &
   static const int slots = resident_slots(kernel);
   Plan p;
   if (!resident_tiling(a.plan, NV, slots, p)) return false;
-  const ResidentWorkspace r = resident_fwd_ws(a.ws, p);
+  ResidentWorkspace r = resident_fwd_ws(a.ws, p);
+  arm_generation(r, a.stream);
   ProfileScope s(kKindFusedFwd, a.stream);
   hipLaunchKernelGGL(kernel, tile_grid(p, 0), dim3(kBlock), 0, a.stream, (const elem_t *)a.x, (elem_t *)a.y, r.sync, a.w, a.b,
                      a.mean, a.rstd, a.sdtype, (A)a.eps, p);
@@ -166,7 +187,8 @@ template <typename PT, int ACT, int NV> bool try_resident_bwd_nv(const BwdArgs &
   static const int slots = resident_slots(kernel);
   Plan p;
   if (!resident_tiling(a.plan, NV, slots, p)) return false;
-  const ResidentWorkspace r = resident_bwd_ws(a.ws, p);
+  ResidentWorkspace r = resident_bwd_ws(a.ws, p);
+  arm_generation(r, a.stream);
   ProfileScope s(kKindFusedBwd, a.stream);
   hipLaunchKernelGGL(kernel, tile_grid(p, 0), dim3(kBlock), 0, a.stream, (const elem_t *)a.x, (const elem_t *)a.dy,
                      (elem_t *)a.dx, a.mean, a.rstd, a.sdtype, a.w, a.b, r.partC, r.sync, a.dw, a.db, p);

@@ -24,6 +24,8 @@ SYMBOLS = (
     "gnnhwc_profile_enable",
     "gnnhwc_profile_collect",
     "gnnhwc_kernel_kind_name",
+    "gnnhwc_set_resident",
+    "gnnhwc_debug_read_trace",
 )
 
 
@@ -52,6 +54,10 @@ def _load():
     lib.gnnhwc_profile_enable.restype = ci
     lib.gnnhwc_profile_collect.argtypes = [ctypes.POINTER(i64), ctypes.POINTER(dbl)]
     lib.gnnhwc_profile_collect.restype = ci
+    lib.gnnhwc_set_resident.argtypes = [ci]
+    lib.gnnhwc_set_resident.restype = ci
+    lib.gnnhwc_debug_read_trace.argtypes = [vp, i64]
+    lib.gnnhwc_debug_read_trace.restype = ci
     lib.gnnhwc_kernel_kind_name.argtypes = [ci]
     lib.gnnhwc_kernel_kind_name.restype = ctypes.c_char_p
     return lib
@@ -71,6 +77,11 @@ def check(rc, what):
 
 def kernel_kind_names():
     return [lib.gnnhwc_kernel_kind_name(k).decode() for k in range(NUM_KERNEL_KINDS)]
+
+
+def set_resident(on):
+    """Allow (True) or forbid (False) the single-launch kernels; returns the previous setting."""
+    return bool(lib.gnnhwc_set_resident(1 if on else 0))
 
 
 def profile_enable(on):

@@ -149,7 +149,10 @@ class GN_NHWC_Func(torch.autograd.Function):
     @staticmethod
     def forward(ctx, X, weight, bias, G, eps, activation):
         ctx.x_shape = X.shape
-        X_flat = X.view(X.shape[0], X.shape[1], -1)
+        R = 1
+        for d in X.shape[2:]:
+            R *= d
+        X_flat = X.view(X.shape[0], X.shape[1], R)  # explicit R: "-1" is ambiguous for an empty batch
         X_out, means, rstds = torch.ops.gnop.fwd(X_flat, weight, bias, G, eps, activation)
         ctx.save_for_backward(X_flat, weight, bias, means, rstds)
         ctx.G = G
@@ -164,7 +167,7 @@ class GN_NHWC_Func(torch.autograd.Function):
         # permuting the channel axis to the end and back works for any rank >= 3.
         nd = dy.dim()
         dy_last = dy.permute(0, *range(2, nd), 1).contiguous()
-        dy_flat = dy_last.view(dy_last.shape[0], -1, dy_last.shape[-1]).permute(0, 2, 1)
+        dy_flat = dy_last.view(X_flat.shape[0], X_flat.shape[2], X_flat.shape[1]).permute(0, 2, 1)
         assert dy_flat.stride() == X_flat.stride() or X_flat.numel() == 0 or 1 in X_flat.shape
         dx, dgamma, dbeta = torch.ops.gnop.bwd(dy_flat, X_flat, weight, bias, means, rstds, ctx.G, ctx.activation)
         return dx.view(ctx.x_shape), dgamma, dbeta, None, None, None

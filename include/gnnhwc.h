@@ -105,6 +105,16 @@ int gnnhwc_bwd(const void *dy, const void *x, const void *weight, const void *bi
                void *workspace, size_t workspace_bytes, void *stream /* hipStream_t */);
 
 /*
+ * Kernel selection (no counterpart in the reference).  By default a problem whose tensors fit in the
+ * register files of one launch is run by the single-launch kernels (x and dy are read from memory once;
+ * workgroups exchange partial results while resident), anything else by the multi-launch streaming
+ * kernels.  The single-launch kernels assume no second such launch is running on another stream of the
+ * same device at the same time; gnnhwc_set_resident(0) (or GNNHWC_DISABLE_RESIDENT=1 in the environment)
+ * forces the streaming kernels.  Process-wide; returns the previous setting.
+ */
+int gnnhwc_set_resident(int on);
+
+/*
  * Per-kernel timing for benchmarks (no counterpart in the reference, which relies on an external
  * profiler, prof.py:1-39).  While enabled, every kernel the library launches on this thread is
  * bracketed by HIP events on the launch stream.  gnnhwc_profile_collect synchronises those events and

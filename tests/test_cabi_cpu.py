@@ -1,0 +1,127 @@
+"""CPU-only checks of the boundary: the shared library loads, exports every symbol include/gnnhwc.h
+declares, sizes workspaces, rejects bad arguments without launching anything, and the Python surface
+mirrors the reference's (src/gnnhwc/custom_gn.py:29-90)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import gnnhwc
+from gnnhwc import GN_NHWC, GN_NHWC_Func, _cabi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "gnnhwc.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(gnnhwc_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_functions()
+    assert {"gnnhwc_fwd", "gnnhwc_bwd", "gnnhwc_fwd_workspace_bytes", "gnnhwc_bwd_workspace_bytes", "gnnhwc_last_error",
+            "gnnhwc_version", "gnnhwc_profile_enable", "gnnhwc_profile_collect", "gnnhwc_kernel_kind_name",
+            "gnnhwc_debug_read_trace", "gnnhwc_set_resident"} <= set(names)
+    lib = ctypes.CDLL(_cabi.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), n
+
+
+def test_version_and_kind_names():
+    assert _cabi.lib.gnnhwc_version() >> 16 == 1
+    names = _cabi.kernel_kind_names()
+    assert len(names) == _cabi.NUM_KERNEL_KINDS and all(names)
+
+
+@pytest.mark.parametrize("dtype", [0, 1, 2, 3])
+def test_workspace_sizes(dtype):
+    lib = _cabi.lib
+    for (N, R, C, G) in [(1, 16384, 640, 32), (4, 16384, 320, 32), (1, 262144, 128, 32), (3, 1961, 96, 24), (8, 289, 1920, 32),
+                         (1, 1, 1, 1), (2, 5, 7, 7)]:
+        f = lib.gnnhwc_fwd_workspace_bytes(N, R, C, G, dtype)
+        b = lib.gnnhwc_bwd_workspace_bytes(N, R, C, G, dtype)
+        assert f > 0 and f % 256 == 0, (N, R, C, G, f)
+        assert b > 0 and b % 256 == 0, (N, R, C, G, b)
+        # scratch stays a small fraction of the tensors it serves
+        S = N * R * C * (8 if dtype == 1 else 4 if dtype == 0 else 2)
+        assert f < 16 * 2 ** 20 and b < 48 * 2 ** 20, (N, R, C, G, f, b, S)
+    assert lib.gnnhwc_fwd_workspace_bytes(0, 16, 8, 2, dtype) == 256  # empty batch
+    assert lib.gnnhwc_fwd_workspace_bytes(1, 16, 7, 3, dtype) == 0
+    assert "divisible" in _cabi.last_error()
+    assert lib.gnnhwc_fwd_workspace_bytes(1, 16, 8, 2, 9) == 0
+    assert "dtype" in _cabi.last_error()
+
+
+def test_invalid_arguments_are_rejected_before_any_launch():
+    lib = _cabi.lib
+    null = None
+    # C % G != 0
+    rc = lib.gnnhwc_fwd(null, null, null, null, null, null, 1, 16, 7, 3, 1e-5, 0, 0, 0, 0, null, 0, null)
+    assert rc == -1 and "divisible" in _cabi.last_error()
+    # unknown activation
+    rc = lib.gnnhwc_fwd(null, null, null, null, null, null, 1, 16, 8, 2, 1e-5, 7, 0, 0, 0, null, 0, null)
+    assert rc == -1 and "activation" in _cabi.last_error()
+    # parameter dtype that may not differ from the data dtype
+    rc = lib.gnnhwc_fwd(null, null, null, null, null, null, 1, 16, 8, 2, 1e-5, 0, 0, 3, 0, null, 0, null)
+    assert rc == -1 and "weight/bias dtype" in _cabi.last_error()
+    rc = lib.gnnhwc_bwd(null, null, null, null, null, null, null, null, null, 1, 16, 8, 2, 0, 2, 2, 1, null, 0, null)
+    assert rc == -1 and "mean/rstd dtype" in _cabi.last_error()
+    # null tensors
+    rc = lib.gnnhwc_fwd(null, null, null, null, null, null, 1, 16, 8, 2, 1e-5, 0, 0, 0, 0, null, 0, null)
+    assert rc == -1 and "null" in _cabi.last_error()
+    # workspace too small (non-null dummy pointers; nothing is dereferenced or launched)
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    rc = lib.gnnhwc_fwd(p, null, null, p, p, p, 1, 16, 8, 2, 1e-5, 0, 0, 0, 0, p, 16, null)
+    assert rc == -2 and "workspace" in _cabi.last_error()
+    rc = lib.gnnhwc_bwd(p, p, null, null, p, p, p, null, null, 1, 16, 8, 2, 0, 0, 0, 0, null, 0, null)
+    assert rc == -2
+    with pytest.raises(RuntimeError):
+        _cabi.check(rc, "gnnhwc_bwd")
+
+
+def test_python_surface_matches_the_reference():
+    assert gnnhwc.GN_NHWC is GN_NHWC and gnnhwc.GN_NHWC_Func is GN_NHWC_Func
+    m = GN_NHWC(4, 8, activation="silu", eps=1e-6)
+    assert isinstance(m, torch.nn.GroupNorm)
+    assert (m.activation, m.act_code, m.eps) == ("silu", 2, 1e-6)
+    assert {k: GN_NHWC(1, 2, activation=k).act_code for k in ("identity", "relu", "swish", "silu", "gelu", "gelu_tanh")} == {
+        "identity": 0, "relu": 1, "swish": 2, "silu": 2, "gelu": 3, "gelu_tanh": 4}
+    assert repr(m) == "GN_NHWC(4, 8, eps=1e-06, affine=True, activation=silu)"
+    assert sorted(m.state_dict()) == ["bias", "weight"]  # loads nn.GroupNorm checkpoints unchanged
+    with pytest.raises(KeyError):
+        GN_NHWC(4, 8, activation="tanh")
+    with pytest.raises(ValueError):
+        GN_NHWC(3, 8)
+    assert GN_NHWC(2, 4, affine=False).weight is None
+
+
+def test_ops_are_registered_and_reject_host_tensors():
+    x = torch.zeros(1, 8, 4).permute(0, 2, 1).contiguous().permute(0, 2, 1)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        torch.ops.gnop.fwd(x, torch.ones(8), torch.zeros(8), 4, 1e-5, 0)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        torch.ops.gnop.bwd(x, x, torch.ones(8), torch.zeros(8), torch.zeros(1, 4), torch.ones(1, 4), 4, 0)
+    # a channels-last CPU tensor reaches the device check through the module as well
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        GN_NHWC(4, 8)(torch.zeros(1, 8, 2, 2).to(memory_format=torch.channels_last))
+
+
+@pytest.mark.parametrize("act", ["identity", "relu", "silu", "gelu", "gelu_tanh"])
+def test_channels_first_input_takes_the_torch_fallback(act):
+    """custom_gn.py:75-79: NCHW input never reaches the kernels, so this path runs on the CPU."""
+    from oracle import gn_oracle as orc
+
+    torch.manual_seed(1)
+    m = GN_NHWC(4, 8, activation=act)
+    x = torch.randn(2, 8, 3, 5, requires_grad=True)
+    y = m(x)
+    want = orc.torch_act(act)(torch.nn.functional.group_norm(x, 4, m.weight, m.bias, m.eps))
+    assert torch.allclose(y, want, rtol=1e-6, atol=1e-7)
+    y.sum().backward()
+    assert x.grad is not None and m.weight.grad is not None
+    m2 = GN_NHWC(4, 8, activation=act, affine=False)
+    assert torch.allclose(m2(x), orc.torch_act(act)(torch.nn.functional.group_norm(x, 4, None, None, m2.eps)), rtol=1e-5, atol=1e-6)
