@@ -50,6 +50,11 @@ __device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
 // unpack / pack convert to and from the accumulation type.
 template <typename T, int VEC> struct LaneVec;
 
+// Makes a register value opaque to the optimiser.  A kernel that keeps packed rows in registers across
+// several passes unpacks them again in every pass; without this the unpacked copies of one pass are
+// kept alive for the next, which doubles or triples the registers a 16-bit tile needs.
+template <typename R> __device__ __forceinline__ void pin(R &r) { asm volatile("" : "+v"(r)); }
+
 template <> struct LaneVec<float, 4> {
   typedef f32x4 raw_t;
   static __device__ __forceinline__ raw_t load(const float *p) { return *(const raw_t *)p; }

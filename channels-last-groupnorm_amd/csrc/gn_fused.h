@@ -178,7 +178,7 @@ __device__ __forceinline__ void wait_flags(const SyncArea &s, int64_t first, int
 //   records : {mean, M2, epoch} per (n, chunk, group, tile)
 // ---------------------------------------------------------------------------------------------
 template <typename T, typename PT, int VEC, int ACT, int NV>
-__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 16 ? 4 : 2))) void fused_fwd_kernel(
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 8 ? 4 : NV <= 16 ? 3 : 2))) void fused_fwd_kernel(
     const T *__restrict__ x, T *__restrict__ y, SyncArea sync_arg, const void *w, const void *b, void *mean_out,
     void *rstd_out, int sdtype, acc_t<T> eps, Plan p) {
   using A = acc_t<T>;
@@ -190,42 +190,41 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 16
   const int64_t n = blockIdx.z;
   const LanePos l = lane_pos(p, n, false);
   const int rows = l.rows;
-  const int rows_blk = (l.len + p.rpi - 1) / p.rpi;  // most rows any lane of this workgroup owns (<= NV)
   const int64_t off = (n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC;
   const int64_t step = (int64_t)p.rpi * p.C;
   typename LV::raw_t buf[NV];
   trace_point(sync, 0);
   if (rows > 0) {
+    // every load is unconditional (rows past the lane's last one re-read it): the waits that follow can then
+    // count loads exactly, and row u is processed while rows u + 1 ... are still in flight
 #pragma unroll
-    for (int u = 0; u < NV; ++u)
-      if (u < rows_blk) buf[u] = LV::load(x + off + (int64_t)clamp_row(u, rows) * step);
+    for (int u = 0; u < NV; ++u) buf[u] = LV::load(x + off + (int64_t)clamp_row(u, rows) * step);
   }
+  A sa[VEC], sb[VEC];
+  if (rows > 0) lane_params<A, PT, VEC>(l, w, b, sa, sb);  // needed after the exchange; in flight until then
   A mean[VEC], m2[VEC];
 #pragma unroll
   for (int j = 0; j < VEC; ++j) { mean[j] = (A)0; m2[j] = (A)0; }
   if (rows > 0) {
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
-      if (u < rows_blk) {
-        const A keep = u < rows ? (A)1 : (A)0;
-        A v[VEC];
-        LV::unpack(buf[u], v);
+      const A keep = u < rows ? (A)1 : (A)0;
+      A v[VEC];
+      LV::unpack(buf[u], v);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) mean[j] += keep * v[j];
-      }
+      for (int j = 0; j < VEC; ++j) mean[j] += keep * v[j];
     }
     const A inv = fast_rcp((A)rows);
 #pragma unroll
     for (int j = 0; j < VEC; ++j) mean[j] *= inv;
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
-      if (u < rows_blk) {
-        const A keep = u < rows ? (A)1 : (A)0;
-        A v[VEC];
-        LV::unpack(buf[u], v);
+      const A keep = u < rows ? (A)1 : (A)0;
+      A v[VEC];
+      pin(buf[u]);
+      LV::unpack(buf[u], v);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) { const A d = v[j] - mean[j]; m2[j] += keep * d * d; }
-      }
+      for (int j = 0; j < VEC; ++j) { const A d = v[j] - mean[j]; m2[j] += keep * d * d; }
     }
   }
   const __amdgpu_buffer_rsrc_t rb = record_buffer(sync);
@@ -279,16 +278,17 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 16
   }
   trace_point(sync, 3);
   if (rows > 0) {
-    A sa[VEC], sb[VEC], unused1[VEC], unused2[VEC];
-    lane_coeffs<A, PT, VEC, false>(p, l, w, b, sm0, sm1, nullptr, nullptr, sa, sb, unused1, unused2);
+    A unused1[VEC], unused2[VEC];
+    lane_coeffs<A, VEC, false>(p, l, sm0, sm1, nullptr, nullptr, sa, sb, unused1, unused2);
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
-      if (u < rows_blk) {
+      if (u < rows) {
         A v[VEC];
+        pin(buf[u]);
         LV::unpack(buf[u], v);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) v[j] = act_fwd<ACT, A>(v[j] * sa[j] + sb[j]);
-        LV::store(y + off + (int64_t)clamp_row(u, rows) * step, LV::pack(v));
+        LV::store(y + off + (int64_t)u * step, LV::pack(v));
       }
     }
   }
@@ -316,7 +316,6 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
   const LanePos l = lane_pos(p, n, false);
   const __amdgpu_buffer_rsrc_t rb = record_buffer(sync);
   const int rows = l.rows;
-  const int rows_blk = (l.len + p.rpi - 1) / p.rpi;
   const int64_t off = (n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC;
   const int64_t step = (int64_t)p.rpi * p.C;
   typename LV::raw_t bx[NV], bd[NV];
@@ -324,36 +323,33 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
   if (rows > 0) {
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
-      if (u < rows_blk) {
-        const int64_t o = off + (int64_t)clamp_row(u, rows) * step;
-        bx[u] = LV::load(x + o);
-        bd[u] = LV::load(dy + o);
-      }
+      const int64_t o = off + (int64_t)clamp_row(u, rows) * step;
+      bx[u] = LV::load(x + o);
+      bd[u] = LV::load(dy + o);
     }
   }
+  A sa[VEC], sb[VEC], c1[VEC], c2[VEC];
+  if (rows > 0) lane_params<A, PT, VEC>(l, w, b, sa, sb);
   stage_chunk_stats<A>(mean, rstd, sdtype, p, l, sm_mu, sm_rs);
   __syncthreads();
   trace_point(sync, 1);
-  A sa[VEC], sb[VEC], c1[VEC], c2[VEC];
   {
     A s1[VEC], s2[VEC];
 #pragma unroll
     for (int j = 0; j < VEC; ++j) { s1[j] = (A)0; s2[j] = (A)0; }
     if (rows > 0) {
-      lane_coeffs<A, PT, VEC, false>(p, l, w, b, sm_mu, sm_rs, nullptr, nullptr, sa, sb, c1, c2);
+      lane_coeffs<A, VEC, false>(p, l, sm_mu, sm_rs, nullptr, nullptr, sa, sb, c1, c2);
 #pragma unroll
       for (int u = 0; u < NV; ++u) {
-        if (u < rows_blk) {
-          const A keep = u < rows ? (A)1 : (A)0;
-          A vx[VEC], vd[VEC];
-          LV::unpack(bx[u], vx);
-          LV::unpack(bd[u], vd);
+        const A keep = u < rows ? (A)1 : (A)0;
+        A vx[VEC], vd[VEC];
+        LV::unpack(bx[u], vx);
+        LV::unpack(bd[u], vd);
 #pragma unroll
-          for (int j = 0; j < VEC; ++j) {
-            const A g = keep * vd[j] * act_bwd<ACT, A>(vx[j] * sa[j] + sb[j]);
-            s1[j] += g * vx[j];
-            s2[j] += g;
-          }
+        for (int j = 0; j < VEC; ++j) {
+          const A g = keep * vd[j] * act_bwd<ACT, A>(vx[j] * sa[j] + sb[j]);
+          s1[j] += g * vx[j];
+          s2[j] += g;
         }
       }
     }
@@ -431,8 +427,10 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
     }
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
-      if (u < rows_blk) {
+      if (u < rows) {
         A vx[VEC], vd[VEC];
+        pin(bx[u]);
+        pin(bd[u]);
         LV::unpack(bx[u], vx);
         LV::unpack(bd[u], vd);
 #pragma unroll
@@ -440,7 +438,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
           const A g = vd[j] * act_bwd<ACT, A>(vx[j] * sa[j] + sb[j]);
           vd[j] = sa[j] * g + (c1[j] * vx[j] + c2[j]);
         }
-        LV::store(dx + off + (int64_t)clamp_row(u, rows) * step, LV::pack(vd));
+        LV::store(dx + off + (int64_t)u * step, LV::pack(vd));
       }
     }
   }

@@ -77,13 +77,17 @@ bool resident_enabled();
 // Device buffer for in-kernel timestamps when GNNHWC_TRACE=1, else null.
 unsigned long long *trace_buffer();
 
-// Consumers merge the tile partials of their own groups unless that would be more than
-// kMaxInlineEntries entries per workgroup; then a compaction kernel runs in between.
+// Consumers merge the tile partials of their own groups in their prologue when every lane has at most kEarly
+// entries to fetch; otherwise a compaction kernel runs in between and leaves one entry per group.
 inline bool needs_compaction(const Plan &p) {
   const int chunk_channels = p.lpr * p.vec;
   const int64_t per_group = (int64_t)p.tiles * ((p.D - 1) / chunk_channels + 2);
-  return per_group * p.gmax > kMaxInlineEntries;
+  const int lanes = merge_lanes_for(p.gmax);
+  return lanes < 1 || per_group > (int64_t)kEarly * lanes;
 }
+// Whether a chunk's groups fit one merge round at all (more than kBlock groups per chunk do not; those plans
+// use the general looping merge).
+inline bool one_round_merge(const Plan &p) { return pow2_at_least(p.gmax) <= kBlock; }
 
 // Bracket one kernel launch with HIP events when profiling is enabled on this thread (gn_api.hip).
 void profile_before(int kind, hipStream_t stream);

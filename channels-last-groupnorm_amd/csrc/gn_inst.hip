@@ -72,31 +72,19 @@ template <typename K> int resident_slots(K kernel) {
   return slots < kMaxResidentBlocks ? slots : kMaxResidentBlocks;
 }
 
-// Choose the row tiling of a resident launch: rows per lane <= nv, all workgroups resident, and the
-// workgroups spread as evenly over the CUs as the shape allows.  Returns false if it does not fit.
+// Row tiling of a resident launch with a register capacity of nv rows per lane: tiles of exactly nv rows per
+// lane (all loads useful; only the last tile of a sample may be short), every workgroup resident.
+// Returns false if it does not fit.
 bool resident_tiling(const Plan &base, int nv, int slots, Plan &out) {
   const int64_t columns = base.N * base.nchunk;
   if (slots <= 0 || columns > slots || base.N > 65535) return false;
-  const int64_t tiles_min = (base.R + (int64_t)nv * base.rpi - 1) / ((int64_t)nv * base.rpi);
-  const int64_t tiles_max = slots / columns;
-  if (tiles_min > tiles_max) return false;
-  int64_t best = -1;
-  double best_eff = -1.0;
-  for (int64_t t = tiles_min; t <= tiles_max; ++t) {
-    int64_t rows = (base.R + t - 1) / t;
-    rows = (rows + base.rpi - 1) / base.rpi * base.rpi;
-    if ((base.R + rows - 1) / rows != t) continue;  // this tile count cannot be realised with equal tiles
-    const int64_t blocks = columns * t;
-    const double eff = (double)blocks / (double)((blocks + kNumCU - 1) / kNumCU * kNumCU);
-    if (eff > best_eff + 1e-9) { best_eff = eff; best = t; }
-  }
-  if (best < 0) return false;
+  const int64_t rows = (int64_t)nv * base.rpi;
+  const int64_t tiles = (base.R + rows - 1) / rows;
+  if (columns * tiles > slots) return false;
   out = base;
-  int64_t rows = (base.R + best - 1) / best;
-  rows = (rows + base.rpi - 1) / base.rpi * base.rpi;
   out.tile_rows = (int)rows;
-  out.tiles = (int)best;
-  out.nblocks = columns * best;
+  out.tiles = (int)tiles;
+  out.nblocks = columns * tiles;
   return true;
 }
 

@@ -71,18 +71,33 @@ __device__ __forceinline__ LanePos lane_pos(const Plan &p, int64_t n, bool rever
 // Row u of batch b is the lane's row min(b U + u, rows - 1): the trailing batch re-reads the last row
 // instead of branching, consumers that accumulate weight such duplicates with 0, consumers that store
 // simply store the same values again.
+// `nb` must be uniform over the workgroup (lanes with fewer rows clamp), and every issue inside the steady
+// state is unconditional: a load issued under a branch would force the waits that follow the join to
+// assume it may not have happened, i.e. to drain the queue, and the two batches would no longer overlap.
 template <typename ISSUE, typename CONSUME>
 __device__ __forceinline__ void double_buffered(int nb, ISSUE &&issue, CONSUME &&consume) {
   using B0 = std::integral_constant<int, 0>;
   using B1 = std::integral_constant<int, 1>;
-  for (int b = 0; b < nb; b += 2) {
-    if (b + 1 < nb) issue(B1{}, b + 1);
+  int b = 0;
+  while (b + 2 < nb) {
+    issue(B1{}, b + 1);
     consume(B0{}, b);
-    if (b + 1 < nb) {
-      if (b + 2 < nb) issue(B0{}, b + 2);
-      consume(B1{}, b + 1);
-    }
+    issue(B0{}, b + 2);
+    consume(B1{}, b + 1);
+    b += 2;
   }
+  if (nb - b == 2) {
+    issue(B1{}, b + 1);
+    consume(B0{}, b);
+    consume(B1{}, b + 1);
+  } else if (nb - b == 1) {
+    consume(B0{}, b);
+  }
+}
+// Batches every active lane of the workgroup walks: the lane rows with the most rows set the count.
+template <int U> __device__ __forceinline__ int block_batches(const Plan &p, const LanePos &l) {
+  const int rows_blk = (l.len + p.rpi - 1) / p.rpi;
+  return (rows_blk + U - 1) / U;
 }
 __device__ __forceinline__ int clamp_row(int idx, int rows) { return idx < rows ? idx : rows - 1; }
 
@@ -123,9 +138,77 @@ __device__ __forceinline__ void group_chunks(const PartialGeo &q, int D, int g, 
   k_lo = (g * D) / q.chunk_channels;
   nk = ((g + 1) * D - 1) / q.chunk_channels - k_lo + 1;
 }
-// Lanes per group for a consumer's merge of tile partials.
+// Lanes per group for a consumer's looping merge of tile partials (general path).
 __device__ __forceinline__ int merge_lanes(const PartialGeo &q, int D) {
   return pow2_ceil_clamped(q.tiles * ((D - 1) / q.chunk_channels + 2), 64);
+}
+
+// Early fetch of tile partials: every group of the chunk gets `L` lanes in a single round, and each lane
+// loads its (at most kEarly) entries of NF fields into registers.  The loads are issued before the lane's
+// first data loads, so they are not queued behind them; they are consumed after those loads are in flight.
+template <typename A, int NF> struct EarlyPartials {
+  A v[kEarly][NF];
+  int L, gi, sl, P;
+  bool valid;
+};
+template <typename A, int NF, bool COH>
+__device__ __forceinline__ void fetch_partials(EarlyPartials<A, NF> &e, const A *__restrict__ part, int64_t plane,
+                                               const PartialGeo &q, const Plan &p, const LanePos &l) {
+  int gp = 1;
+  while (gp < p.gmax) gp <<= 1;
+  e.L = kBlock / gp < 64 ? kBlock / gp : 64;
+  e.gi = threadIdx.x / e.L;
+  e.sl = threadIdx.x % e.L;
+  e.valid = e.gi < l.ng;
+  const int g = l.g_lo + e.gi;
+  int k_lo = 0, nk = 1;
+  if (e.valid) group_chunks(q, p.D, g, k_lo, nk);
+  e.P = e.valid ? q.tiles * nk : 0;
+  const int64_t base = group_slot(q, p.G, l.n, 0, k_lo, g);
+  const int64_t kstride = (int64_t)p.G * q.tiles;
+#pragma unroll
+  for (int i = 0; i < kEarly; ++i) {
+    const int en = e.sl + i * e.L;
+    const bool have = en < e.P;
+    const int k = have ? en / q.tiles : 0, t = have ? en - k * q.tiles : 0;
+    const int64_t slot = base + k * kstride + t;
+#pragma unroll
+    for (int f = 0; f < NF; ++f) e.v[i][f] = have ? ld_part<COH>(part + f * plane + slot) : (A)0;
+  }
+}
+// (count, mean, M2) entries -> merged triple (pivot form), available in every lane of the group's segment.
+template <typename A> __device__ __forceinline__ Moments<A> reduce_moments(const EarlyPartials<A, 3> &e) {
+  A nl = (A)0, s1 = (A)0, s2 = (A)0;
+  const A kl = e.v[0][1];
+#pragma unroll
+  for (int i = 0; i < kEarly; ++i) {
+    const A cn = e.v[i][0];
+    const A d = e.v[i][1] - kl;
+    nl += cn;
+    s1 += cn * d;
+    s2 += e.v[i][2] + cn * d * d;
+  }
+  const A inv = nl > (A)0 ? (A)1 / nl : (A)0;
+  const A mean_l = kl + s1 * inv;
+  const A m2_l = s2 - s1 * s1 * inv;
+  const A K = __shfl(mean_l, (int)(threadIdx.x & 63 & ~(e.L - 1)), 64);
+  const A d = mean_l - K;
+  A t0 = nl, t1 = nl * d, t2 = m2_l + nl * d * d;
+  t0 = segment_sum(t0, e.L);
+  segment_sum2(t1, t2, e.L);
+  Moments<A> r;
+  r.n = t0;
+  const A dm = e.valid ? t1 / t0 : (A)0;
+  r.mean = K + dm;
+  r.m2 = t2 - t1 * dm;
+  return r;
+}
+template <typename A> __device__ __forceinline__ void reduce_sums(const EarlyPartials<A, 2> &e, A &ta, A &tb) {
+  ta = (A)0;
+  tb = (A)0;
+#pragma unroll
+  for (int i = 0; i < kEarly; ++i) { ta += e.v[i][0]; tb += e.v[i][1]; }
+  segment_sum2(ta, tb, e.L);
 }
 // Channels [ca, cb) (relative to the chunk) of group g that lie inside the chunk.
 __device__ __forceinline__ void group_span(const Plan &p, const LanePos &l, int g, int &ca, int &cb) {
@@ -186,7 +269,8 @@ __device__ __forceinline__ void lane_stats(const T *__restrict__ x, const Plan &
   for (int j = 0; j < VEC; ++j) { mean[j] = (A)0; m2[j] = (A)0; }
   A cnt = (A)0;
   const int rows = l.rows;
-  const int nb = (rows + U - 1) / U;
+  const int nb = block_batches<U>(p, l);
+  if (rows == 0) return;
   const T *base = x + ((l.n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC);
   const int64_t step = (int64_t)p.rpi * p.C;
   typename LV::raw_t buf0[U], buf1[U];
@@ -199,11 +283,13 @@ __device__ __forceinline__ void lane_stats(const T *__restrict__ x, const Plan &
     }
   };
   auto consume = [&](auto sel, int b) {
-    const int m = rows - b * U < U ? rows - b * U : U;
+    int m = rows - b * U;
+    m = m < 0 ? 0 : (m > U ? U : m);
+    if (m == 0) return;  // only in the last batch of a lane row that is one row short
     if constexpr (decltype(sel)::value == 0) fold_batch<T, VEC, U>(buf0, m, cnt, mean, m2);
     else fold_batch<T, VEC, U>(buf1, m, cnt, mean, m2);
   };
-  if (nb > 0) issue(std::integral_constant<int, 0>{}, 0);
+  issue(std::integral_constant<int, 0>{}, 0);
   double_buffered(nb, issue, consume);
 }
 
@@ -361,7 +447,7 @@ __device__ __forceinline__ void block_channel_sums(const Plan &p, const LanePos 
 //   part : 3 planes [N][nchunk][G][tiles]; only the groups a chunk intersects are written.
 // ---------------------------------------------------------------------------------------------
 template <typename T, int VEC>
-__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) void stats_kernel(
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) void stats_kernel(
     const T *__restrict__ x, acc_t<T> *__restrict__ part, Plan p) {
   using A = acc_t<T>;
   __shared__ A sm_mean[kBlock * VEC];
@@ -382,7 +468,9 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) voi
 }
 
 // Merge the P = tiles * (chunks holding a piece of g) partial triples of group g with `L` lanes; every
-// lane of the segment returns the merged triple (exact two-pass form).
+// lane of the segment returns the merged triple.  One pass over the entries (all loads independent, one
+// memory round trip): each lane folds its entries about the mean of its first one, then the lanes are
+// merged about the first lane's mean (the pivot form of the two-pass merge).
 template <typename A, bool COH>
 __device__ __forceinline__ Moments<A> merge_group_partials(const A *__restrict__ part, int64_t plane, const PartialGeo &q,
                                                            int G, int D, int64_t n, int g, bool valid, int L, int sl) {
@@ -392,27 +480,32 @@ __device__ __forceinline__ Moments<A> merge_group_partials(const A *__restrict__
   // entries of chunk k_lo .. k_lo + nk - 1 are contiguous runs of q.tiles values each
   const int64_t base = group_slot(q, G, n, 0, k_lo, g);
   const int64_t kstride = (int64_t)G * q.tiles;
-  A sn = (A)0, sm = (A)0;
+  A nl = (A)0, kl = (A)0, s1 = (A)0, s2 = (A)0;
   for (int e = sl; e < P; e += L) {
     const int k = e / q.tiles, t = e - k * q.tiles;
     const int64_t slot = base + k * kstride + t;
     const A cn = ld_part<COH>(part + slot);
-    sn += cn;
-    sm += cn * ld_part<COH>(part + plane + slot);
+    const A mu = ld_part<COH>(part + plane + slot);
+    const A mm = ld_part<COH>(part + 2 * plane + slot);
+    if (nl == (A)0) kl = mu;
+    const A d = mu - kl;
+    nl += cn;
+    s1 += cn * d;
+    s2 += mm + cn * d * d;
   }
-  sn = segment_sum(sn, L);
-  sm = segment_sum(sm, L);
+  const A inv = nl > (A)0 ? (A)1 / nl : (A)0;
+  const A mean_l = kl + s1 * inv;
+  const A m2_l = s2 - s1 * s1 * inv;
+  const A K = __shfl(mean_l, (int)(threadIdx.x & 63 & ~(L - 1)), 64);
+  const A d = mean_l - K;
+  A t0 = nl, t1 = nl * d, t2 = m2_l + nl * d * d;
+  t0 = segment_sum(t0, L);
+  segment_sum2(t1, t2, L);
   Moments<A> r;
-  r.n = sn;
-  r.mean = valid ? sm / sn : (A)0;
-  A s2 = (A)0;
-  for (int e = sl; e < P; e += L) {
-    const int k = e / q.tiles, t = e - k * q.tiles;
-    const int64_t slot = base + k * kstride + t;
-    const A d = ld_part<COH>(part + plane + slot) - r.mean;
-    s2 += ld_part<COH>(part + 2 * plane + slot) + ld_part<COH>(part + slot) * d * d;
-  }
-  r.m2 = segment_sum(s2, L);
+  r.n = t0;
+  const A dm = valid ? t1 / t0 : (A)0;
+  r.mean = K + dm;
+  r.m2 = t2 - t1 * dm;
   return r;
 }
 
@@ -476,15 +569,12 @@ __device__ __forceinline__ void stage_chunk_stats(const void *mean, const void *
   }
 }
 
-// a = rstd * gamma, b = beta - mean * a: normalise + affine as one FMA per element (same folding as
-// src/gnnhwc/csrc/gn_kernel.cu:350-379, 601-602, 783-784).  Group statistics come from LDS; optional
-// per-group extras (the backward's coef1 / coef2) are fetched alongside.
-template <typename A, typename PT, int VEC, bool EXTRA>
-__device__ __forceinline__ void lane_coeffs(const Plan &p, const LanePos &l, const void *w, const void *b,
-                                            const A *sm_mu, const A *sm_rs, const A *sm_c1, const A *sm_c2, A (&sa)[VEC],
-                                            A (&sb)[VEC], A (&c1)[VEC], A (&c2)[VEC]) {
+// gamma / beta of the lane's channels.  Issued early, next to the first data loads, so that their latency
+// is hidden behind whatever the kernel has to wait for anyway.
+template <typename A, typename PT, int VEC>
+__device__ __forceinline__ void lane_params(const LanePos &l, const void *w, const void *b, A (&gamma)[VEC],
+                                            A (&beta)[VEC]) {
   const int c = l.cvi * VEC;
-  A gamma[VEC], beta[VEC];
   if (w) {
 #pragma unroll
     for (int j = 0; j < VEC; ++j) gamma[j] = load_param<PT, A>(w, c + j);
@@ -499,13 +589,22 @@ __device__ __forceinline__ void lane_coeffs(const Plan &p, const LanePos &l, con
 #pragma unroll
     for (int j = 0; j < VEC; ++j) beta[j] = (A)0;
   }
+}
+// a = rstd * gamma, b = beta - mean * a: normalise + affine as one FMA per element (same folding as
+// src/gnnhwc/csrc/gn_kernel.cu:350-379, 601-602, 783-784).  Group statistics come from LDS; optional
+// per-group extras (the backward's coef1 / coef2) are fetched alongside.  On return sa / sb replace gamma / beta.
+template <typename A, int VEC, bool EXTRA>
+__device__ __forceinline__ void lane_coeffs(const Plan &p, const LanePos &l, const A *sm_mu, const A *sm_rs,
+                                            const A *sm_c1, const A *sm_c2, A (&sa)[VEC], A (&sb)[VEC], A (&c1)[VEC],
+                                            A (&c2)[VEC]) {
+  const int c = l.cvi * VEC;
   int gi = c / p.D;
   int rem = c - gi * p.D;
   gi -= l.g_lo;
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
-    sa[j] = sm_rs[gi] * gamma[j];
-    sb[j] = beta[j] - sm_mu[gi] * sa[j];
+    sa[j] = sm_rs[gi] * sa[j];
+    sb[j] = sb[j] - sm_mu[gi] * sa[j];
     if (EXTRA) {
       c1[j] = sm_c1[gi];
       c2[j] = sm_c2[gi];
@@ -523,7 +622,7 @@ __device__ __forceinline__ void lane_coeffs(const Plan &p, const LanePos &l, con
 // whatever type the reported statistics have (cf. gn_kernel.cu:290-291).
 // ---------------------------------------------------------------------------------------------
 template <typename T, typename PT, int VEC, int ACT>
-__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) void apply_kernel(
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) void apply_kernel(
     const T *__restrict__ x, T *__restrict__ y, const acc_t<T> *__restrict__ part, PartialGeo q, const void *w,
     const void *b, void *mean_out, void *rstd_out, int sdtype, acc_t<T> eps, Plan p) {
   using A = acc_t<T>;
@@ -531,10 +630,11 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) voi
   constexpr int U = kUnrollFwd;
   __shared__ A sm_mu[kBlock * VEC];
   __shared__ A sm_rs[kBlock * VEC];
+  const bool one_round = pow2_at_least(p.gmax) <= kBlock;
   for (int64_t n = blockIdx.z; n < p.N; n += gridDim.z) {
     const LanePos l = lane_pos(p, n, true);
     const int rows = l.rows;
-    const int nb = (rows + U - 1) / U;
+    const int nb = block_batches<U>(p, l);
     const int64_t off = (n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC;
     const int64_t step = (int64_t)p.rpi * p.C;
     typename LV::raw_t buf0[U], buf1[U];
@@ -555,13 +655,35 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) voi
         else LV::unpack(buf1[u], v);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) v[j] = act_fwd<ACT, A>(v[j] * sa[j] + sb[j]);
-        LV::store(y + off + (int64_t)clamp_row(bi * U + u, rows) * step, LV::pack(v));
+        if (bi * U + u < rows) LV::store(y + off + (int64_t)(bi * U + u) * step, LV::pack(v));
       }
     };
-    if (nb > 0) issue(std::integral_constant<int, 0>{}, 0);  // in flight while the statistics are merged
-    merge_chunk_stats<A, false>(part, q, p, l, eps, sm_mu, sm_rs, mean_out, rstd_out, sdtype);
-    if (nb > 0) {
-      lane_coeffs<A, PT, VEC, false>(p, l, w, b, sm_mu, sm_rs, nullptr, nullptr, sa, sb, unused1, unused2);
+    // order of issue: the few small loads the prologue depends on first, then the first batch of x, so that
+    // the small ones are not queued behind the bulk traffic of every workgroup
+    EarlyPartials<A, 3> early;
+    if (one_round) fetch_partials<A, 3, false>(early, part, group_plane(q, p.G, p.N), q, p, l);
+    if (rows > 0) {
+      lane_params<A, PT, VEC>(l, w, b, sa, sb);
+      issue(std::integral_constant<int, 0>{}, 0);
+    }
+    if (one_round) {
+      const Moments<A> m = reduce_moments<A>(early);
+      if (early.valid && early.sl == 0) {
+        const int g = l.g_lo + early.gi;
+        const A rs = (A)1 / sqrt(m.m2 / m.n + eps);
+        sm_mu[early.gi] = m.mean;
+        sm_rs[early.gi] = rs;
+        if (l.tile == 0 && g * p.D >= l.cstart) {  // the chunk where the group starts reports it
+          store_scalar<A>(mean_out, n * p.G + g, sdtype, m.mean);
+          store_scalar<A>(rstd_out, n * p.G + g, sdtype, rs);
+        }
+      }
+      __syncthreads();
+    } else {
+      merge_chunk_stats<A, false>(part, q, p, l, eps, sm_mu, sm_rs, mean_out, rstd_out, sdtype);
+    }
+    if (rows > 0) {
+      lane_coeffs<A, VEC, false>(p, l, sm_mu, sm_rs, nullptr, nullptr, sa, sb, unused1, unused2);
       double_buffered(nb, issue, consume);
     }
     __syncthreads();  // sm_mu / sm_rs are rewritten for the next sample of a wrapped grid
@@ -576,7 +698,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) voi
 //   partC : [N][tiles][C][2]      partG : 2 planes [N][nchunk][G][tiles]
 // ---------------------------------------------------------------------------------------------
 template <typename T, typename PT, int VEC, int ACT>
-__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) void bwd_reduce_kernel(
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) void bwd_reduce_kernel(
     const T *__restrict__ x, const T *__restrict__ dy, const void *mean, const void *rstd, int sdtype, const void *w,
     const void *b, acc_t<T> *__restrict__ partC, acc_t<T> *__restrict__ partG, Plan p) {
   using A = acc_t<T>;
@@ -591,7 +713,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) voi
   for (int64_t n = blockIdx.z; n < p.N; n += gridDim.z) {
     const LanePos l = lane_pos(p, n, false);
     const int rows = l.rows;
-    const int nb = (rows + U - 1) / U;
+    const int nb = block_batches<U>(p, l);
     const int64_t off = (n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC;
     const int64_t step = (int64_t)p.rpi * p.C;
     typename LV::raw_t bx0[U], bx1[U], bd0[U], bd1[U];
@@ -619,13 +741,16 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) voi
         }
       }
     };
-    if (nb > 0) issue(std::integral_constant<int, 0>{}, 0);
-    stage_chunk_stats<A>(mean, rstd, sdtype, p, l, sm_mu, sm_rs);
+    stage_chunk_stats<A>(mean, rstd, sdtype, p, l, sm_mu, sm_rs);  // small loads first, then the bulk
+    if (rows > 0) {
+      lane_params<A, PT, VEC>(l, w, b, sa, sb);
+      issue(std::integral_constant<int, 0>{}, 0);
+    }
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < VEC; ++j) { s1[j] = (A)0; s2[j] = (A)0; }
-    if (nb > 0) {
-      lane_coeffs<A, PT, VEC, false>(p, l, w, b, sm_mu, sm_rs, nullptr, nullptr, sa, sb, unused1, unused2);
+    if (rows > 0) {
+      lane_coeffs<A, VEC, false>(p, l, sm_mu, sm_rs, nullptr, nullptr, sa, sb, unused1, unused2);
       double_buffered(nb, issue, consume);
     }
     block_channel_sums<A, VEC>(p, l, s1, s2, sm1, sm2);
@@ -742,13 +867,14 @@ __global__ __launch_bounds__(kBlock) void bwd_compact_kernel(const A *__restrict
 // chunk, dgamma_c = sum_n (S1 - mean S2) rstd and dbeta_c = sum_n S2 (compute_dweight_dbias, gn_kernel.cu:695-728).
 // ---------------------------------------------------------------------------------------------
 template <typename T, typename PT, int VEC, int ACT>
-__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) void bwd_dx_kernel(
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) void bwd_dx_kernel(
     const T *__restrict__ x, const T *__restrict__ dy, T *__restrict__ dx, const void *mean, const void *rstd, int sdtype,
     const void *w, const void *b, const acc_t<T> *__restrict__ partC, const acc_t<T> *__restrict__ partG, PartialGeo q,
     void *dw, void *db, Plan p) {
   using A = acc_t<T>;
   using LV = LaneVec<T, VEC>;
   constexpr int U = kUnrollBwd;
+  const bool one_round = pow2_at_least(p.gmax) <= kBlock;
   __shared__ A sm_c1[kBlock * VEC];
   __shared__ A sm_c2[kBlock * VEC];
   __shared__ A sm_mu[kBlock * VEC];
@@ -796,7 +922,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) voi
   for (int64_t n = blockIdx.z; n < p.N; n += gridDim.z) {
     const LanePos l = lane_pos(p, n, true);
     const int rows = l.rows;
-    const int nb = (rows + U - 1) / U;
+    const int nb = block_batches<U>(p, l);
     const int64_t off = (n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC;
     const int64_t step = (int64_t)p.rpi * p.C;
     typename LV::raw_t bx0[U], bx1[U], bd0[U], bd1[U];
@@ -820,11 +946,34 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) voi
           const A g = vd[j] * act_bwd<ACT, A>(vx[j] * sa[j] + sb[j]);
           vd[j] = sa[j] * g + (c1[j] * vx[j] + c2[j]);
         }
-        LV::store(dx + off + (int64_t)clamp_row(bi * U + u, rows) * step, LV::pack(vd));
+        if (bi * U + u < rows) LV::store(dx + off + (int64_t)(bi * U + u) * step, LV::pack(vd));
       }
     };
-    if (nb > 0) issue(std::integral_constant<int, 0>{}, 0);  // in flight while the group sums are merged
-    {
+    EarlyPartials<A, 2> early;
+    A emu = (A)0, ers = (A)0;
+    if (one_round) {
+      fetch_partials<A, 2, false>(early, partG, plane, q, p, l);
+      if (early.valid && early.sl == 0) {
+        emu = load_scalar<A>(mean, n * p.G + l.g_lo + early.gi, sdtype);
+        ers = load_scalar<A>(rstd, n * p.G + l.g_lo + early.gi, sdtype);
+      }
+    }
+    if (rows > 0) {
+      lane_params<A, PT, VEC>(l, w, b, sa, sb);
+      issue(std::integral_constant<int, 0>{}, 0);  // in flight while the group sums are merged
+    }
+    if (one_round) {
+      A ta, tb;
+      reduce_sums<A>(early, ta, tb);
+      if (early.valid && early.sl == 0) {
+        const A s = (A)1 / ((A)p.D * (A)p.R);
+        const A k1 = (emu * tb - ta) * s * ers * ers * ers;
+        sm_mu[early.gi] = emu;
+        sm_rs[early.gi] = ers;
+        sm_c1[early.gi] = k1;
+        sm_c2[early.gi] = -emu * k1 - tb * s * ers;
+      }
+    } else {
       const int L = merge_lanes(q, p.D);
       const int nseg = kBlock / L;
       const int seg = threadIdx.x / L, sl = threadIdx.x % L;
@@ -847,8 +996,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) voi
       }
     }
     __syncthreads();
-    if (nb > 0) {
-      lane_coeffs<A, PT, VEC, true>(p, l, w, b, sm_mu, sm_rs, sm_c1, sm_c2, sa, sb, c1, c2);
+    if (rows > 0) {
+      lane_coeffs<A, VEC, true>(p, l, sm_mu, sm_rs, sm_c1, sm_c2, sa, sb, c1, c2);
       double_buffered(nb, issue, consume);
     }
     __syncthreads();

@@ -15,7 +15,7 @@ constexpr int kUnrollFwd = 4;       // independent row loads in flight per lane,
 constexpr int kUnrollBwd = 2;       // ... two-input kernels (x and dy)
 constexpr int kNumCU = 256;         // MI355X
 constexpr int kTargetBlocks = 512;  // aim for ~2 workgroups per CU when the tensor is large enough
-constexpr int kMaxInlineEntries = 2048;  // tile partials a consumer workgroup may merge in its prologue
+constexpr int kEarly = 4;            // tile partials a lane of a consumer workgroup fetches ahead of its data
 
 // One workgroup owns `tile_rows` consecutive rows of one sample and one chunk of `lpr` lane vectors
 // (lpr * vec channels) of every such row.  Inside the workgroup thread t handles lane vector
@@ -42,5 +42,18 @@ struct PartialGeo {
   int tiles, nchunk;
   int chunk_channels;  // channels per chunk of the producer (lpr * vec); C when compacted
 };
+
+// A consumer workgroup merges the tile partials of all groups of its chunk in one round: merge_lanes lanes
+// per group, each fetching at most kEarly entries.  The host checks that this covers the plan and
+// otherwise runs the compaction kernel first (which leaves one entry per group).
+__host__ __device__ inline int pow2_at_least(int v) {
+  int p = 1;
+  while (p < v) p <<= 1;
+  return p;
+}
+__host__ __device__ inline int merge_lanes_for(int gmax) {
+  const int l = kBlock / pow2_at_least(gmax);
+  return l > 64 ? 64 : l;
+}
 
 }  // namespace gn
