@@ -9,8 +9,12 @@ inputs, outputs and workspaces already resident in HBM.  The timed region is K s
 torch.cuda.synchronize() calls.  Prints ONE JSON line:
 
   value        algorithmic GB/s of the timed region: (2 S fwd + 3 S bwd per shape) / time
-  roofline     the dominant kernel's algorithmic bytes per launch / its mean duration, measured here with
-               HIP events recorded on the launch stream around every launch, against 8 TB/s
+  roofline     the dominant launch (the kernel kind and shape with the longest mean duration): its algorithmic
+               bytes / its mean duration, measured here with HIP events recorded on the launch stream around
+               every launch, against 8 TB/s; `traffic` is read from profiles/hbm_traffic_sd_unet.txt (rocprofv3
+               --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --counter-workload`), null when that file is absent
+  copy_ceiling the library's plain copy kernel on tensors of each shape's size: what a kernel with no
+               arithmetic and no cross-workgroup dependency reaches at that size on this GPU
   cpu_baseline torch.nn.functional.group_norm + SiLU + autograd on the host cores, same tensors (bounded sample)
   shapes       per-shape us/call and GB/s, with warm (same buffers every call) and cold (rotating through
                > 512 MB of distinct buffers) figures
@@ -43,6 +47,8 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--graph", action="store_true", help="time the replay of a HIP graph of the K steps instead of eager launches")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
+    ap.add_argument("--counter-workload", action="store_true",
+                    help="no timing: one 256 MiB plain copy (calibration) and a few fwd+bwd calls per shape, for a rocprofv3 --pmc run")
     return ap.parse_args()
 
 
@@ -180,21 +186,82 @@ def measure_shape(prob_warm, prob_cold, steps, warmup, use_graph):
 
 
 def kernel_profile(probs, steps):
-    """Mean duration of every kernel kind over `steps` eager steps, from HIP events around each launch."""
+    """{shape: {kind: mean us}} over `steps` eager steps of the whole workload, from HIP events recorded on the
+    launch stream around each launch (the shapes run interleaved, as in the timed region)."""
     import torch
     from gnnhwc import _cabi
 
     stream = torch.cuda.current_stream().cuda_stream
+    acc = {p.cfg.name: {} for p in probs}
     torch.cuda.synchronize()
     _cabi.profile_enable(True)
     try:
         for _ in range(steps):
             for p in probs:
                 p.step(0, stream)
-        res = _cabi.profile_collect()
+                for kind, (n, ms) in _cabi.profile_collect().items():
+                    if n:
+                        a = acc[p.cfg.name].setdefault(kind, [0, 0.0])
+                        a[0] += n
+                        a[1] += ms
     finally:
         _cabi.profile_enable(False)
-    return res
+    return {name: {k: v[1] / v[0] * 1e3 for k, v in kinds.items()} for name, kinds in acc.items()}
+
+
+def copy_ceiling(nbytes, device, steps):
+    """GB/s (read + write) of the library's plain copy kernel on a tensor of nbytes, warm, eager launches."""
+    import torch
+    from gnnhwc import _cabi
+
+    n = (nbytes + 15) // 16 * 16
+    src = torch.empty((n,), dtype=torch.uint8, device=device).random_(0, 255)
+    dst = torch.empty_like(src)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def one():
+        _cabi.check(_cabi.lib.gnnhwc_debug_copy(dst.data_ptr(), src.data_ptr(), n, stream), "gnnhwc_debug_copy")
+
+    t = time_region(one, steps, 10, False, reps=5)
+    return 2 * n / (t / steps) / 1e9
+
+
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_sd_unet.txt")
+
+
+def recorded_traffic():
+    """{(shape, kind): (fetch_bytes, write_bytes)} from the lines `TRAFFIC <shape> <kind> <fetch> <write>` of the
+    committed counter summary, or {} when there is none."""
+    out = {}
+    try:
+        with open(TRAFFIC_FILE) as f:
+            for ln in f:
+                w = ln.split()
+                if len(w) == 5 and w[0] == "TRAFFIC":
+                    out[(w[1], w[2])] = (float(w[3]), float(w[4]))
+    except OSError:
+        pass
+    return out
+
+
+def counter_workload(probs, device):
+    """What `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` observe: a plain copy of known size first (its
+    counter reading calibrates the unit), then every shape's forward and backward a few times."""
+    import torch
+    from gnnhwc import _cabi
+
+    stream = torch.cuda.current_stream().cuda_stream
+    n = 256 << 20
+    src = torch.empty((n,), dtype=torch.uint8, device=device).random_(0, 255)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        _cabi.check(_cabi.lib.gnnhwc_debug_copy(dst.data_ptr(), src.data_ptr(), n, stream), "gnnhwc_debug_copy")
+    torch.cuda.synchronize()
+    for p in probs:
+        for _ in range(5):
+            p.step(0, stream)
+        torch.cuda.synchronize()
+    print(json.dumps({"counter_workload": [p.cfg.name for p in probs], "copy_bytes": n}))
 
 
 def cpu_baseline(cfg_names, seconds):
@@ -260,6 +327,10 @@ def main():
         for p in probs:
             p.step(0, s)
 
+    if args.counter_workload:
+        counter_workload(probs, device)
+        return
+
     # ---- headline: K steps between synchronisations ----
     t = time_region(step, args.steps, args.warmup, use_graph, reps=1)
     alg = sum(p.alg_bytes() for p in probs)
@@ -269,22 +340,29 @@ def main():
 
     # ---- per-kernel durations (HIP events on the launch stream) ----
     prof = kernel_profile(probs, max(20, args.steps // 4))
-    kinds = {k: v for k, v in prof.items() if v[0] > 0}
-    dominant = max(kinds, key=lambda k: kinds[k][1])
-    launches, total_ms = kinds[dominant]
-    mean_S = sum(p.S for p in probs) / len(probs)
-    achieved = KERNEL_STREAMS[dominant] * mean_S / (total_ms / launches * 1e-3) / 1e9
+    S_of = {p.cfg.name: p.S for p in probs}
+    dom_shape, dominant = max(((n, k) for n in prof for k in prof[n]), key=lambda nk: prof[nk[0]][nk[1]])
+    dom_us = prof[dom_shape][dominant]
+    dom_bytes = KERNEL_STREAMS[dominant] * S_of[dom_shape]
+    achieved = dom_bytes / (dom_us * 1e-6) / 1e9
+    traffic = recorded_traffic()
+    tr = traffic.get((dom_shape, dominant))
     roofline = {
         "bound": "hbm",
         "kernel": dominant,
+        "shape": dom_shape,
         "achieved": round(achieved, 1),
         "peak": HBM_PEAK_GBPS,
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBPS, 4),
-        "traffic": None,
-        "bytes_per_launch": KERNEL_STREAMS[dominant] * mean_S,
-        "mean_launch_us": round(total_ms / launches * 1e3, 3),
-        "kernels_us": {k: round(v[1] / v[0] * 1e3, 3) for k, v in kinds.items()},
+        "traffic": round(tr[0] + tr[1]) if tr else None,
+        "traffic_source": "profiles/hbm_traffic_sd_unet.txt (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, copy-calibrated)" if tr else None,
+        "bytes_per_launch": dom_bytes,
+        "mean_launch_us": round(dom_us, 3),
+        "kernels": {n: {k: {"us": round(us, 3), "alg_bytes": KERNEL_STREAMS[k] * S_of[n],
+                            "frac": round(KERNEL_STREAMS[k] * S_of[n] / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+                            "traffic": (round(sum(traffic[(n, k)])) if (n, k) in traffic else None)}
+                        for k, us in kinds.items()} for n, kinds in prof.items()},
     }
 
     # ---- per-shape table ----
@@ -302,6 +380,7 @@ def main():
         key = "fwd_bwd" if cfg.passes != "fwd" else "fwd"
         r["warm_frac_of_peak"] = round(r["warm_%s_gbps" % key] / HBM_PEAK_GBPS, 4)
         r["cold_frac_of_peak"] = round(r["cold_%s_gbps" % key] / HBM_PEAK_GBPS, 4)
+        r["copy_kernel_gbps"] = round(copy_ceiling(S, device, k), 1)
         shapes[n] = r
         del warm, cold
         torch.cuda.empty_cache()

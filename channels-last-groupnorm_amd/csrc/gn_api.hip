@@ -180,6 +180,23 @@ __global__ void fill_zero_kernel(void *p, int64_t n, int dtype) {
   }
 }
 
+// Plain 16-byte-per-lane copy: the yardstick the library's kernels are measured against (same block size,
+// same access width, no arithmetic), and the known-size dispatch that calibrates memory-traffic counters.
+__global__ __launch_bounds__(256) void copy_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, int64_t n16) {
+  const int64_t base = ((int64_t)blockIdx.x * 4) * 256 + threadIdx.x;
+  uint4 v[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int64_t i = base + (int64_t)u * 256;
+    v[u] = src[i < n16 ? i : n16 - 1];
+  }
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int64_t i = base + (int64_t)u * 256;
+    if (i < n16) dst[i] = v[u];
+  }
+}
+
 // ---- per-kernel event timing ----
 struct Timed {
   int kind;
@@ -231,19 +248,17 @@ bool resident_enabled() {
   return v < 0 ? off == 0 : v != 0;
 }
 
-void profile_before(int kind, hipStream_t stream) {
-  if (!g_profile) return;
+bool profile_events(int kind, hipEvent_t *start, hipEvent_t *stop) {
+  if (!g_profile) return false;
   Timed t;
   t.kind = kind;
   t.start = get_event();
   t.stop = get_event();
-  if (!t.start || !t.stop) return;
-  (void)hipEventRecord(t.start, stream);
+  if (!t.start || !t.stop) return false;
   g_timed.push_back(t);
-}
-void profile_after(int kind, hipStream_t stream) {
-  if (!g_profile || g_timed.empty() || g_timed.back().kind != kind) return;
-  (void)hipEventRecord(g_timed.back().stop, stream);
+  *start = t.start;
+  *stop = t.stop;
+  return true;
 }
 
 }  // namespace gn
@@ -388,9 +403,21 @@ int gnnhwc_debug_read_trace(unsigned long long *out, int64_t count) {
   return GNNHWC_OK;
 }
 
+int gnnhwc_debug_copy(void *dst, const void *src, size_t bytes, void *stream) {
+  if (!dst || !src || bytes == 0 || bytes % 16 != 0 || ((uintptr_t)dst | (uintptr_t)src) % 16 != 0)
+    return fail(GNNHWC_ERR_INVALID_ARGUMENT, "copy of %zu bytes: pointers and size must be non-null multiples of 16", bytes);
+  const int64_t n16 = (int64_t)(bytes / 16);
+  const int64_t grid = (n16 + 1023) / 1024;
+  if (grid > 0x7fffffff) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "copy of %zu bytes is too large", bytes);
+  launch(kKindCopy, copy_kernel, dim3((unsigned)grid), dim3(256), (hipStream_t)stream, (const uint4 *)src, (uint4 *)dst, n16);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(GNNHWC_ERR_LAUNCH, "copy launch failed: %s", hipGetErrorString(e));
+  return GNNHWC_OK;
+}
+
 const char *gnnhwc_kernel_kind_name(int kind) {
   static const char *names[GNNHWC_NUM_KERNEL_KINDS] = {"fwd_stats", "fwd_stats_compact", "fwd_apply", "bwd_reduce",
-                                                       "bwd_compact", "bwd_dx", "fused_fwd", "fused_bwd"};
+                                                       "bwd_compact", "bwd_dx", "fused_fwd", "fused_bwd", "copy"};
   return (kind >= 0 && kind < GNNHWC_NUM_KERNEL_KINDS) ? names[kind] : "";
 }
 

@@ -2,6 +2,7 @@
 // (gn_inst.hip, compiled once per type).
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stddef.h>
 #include <stdint.h>
 #include "gn_plan.h"
@@ -17,7 +18,8 @@ enum KernelKind {
   kKindBwdDx = 5,
   kKindFusedFwd = 6,
   kKindFusedBwd = 7,
-  kNumKinds = 8
+  kKindCopy = 8,
+  kNumKinds = 9
 };
 
 struct FwdArgs {
@@ -89,15 +91,19 @@ inline bool needs_compaction(const Plan &p) {
 // use the general looping merge).
 inline bool one_round_merge(const Plan &p) { return pow2_at_least(p.gmax) <= kBlock; }
 
-// Bracket one kernel launch with HIP events when profiling is enabled on this thread (gn_api.hip).
-void profile_before(int kind, hipStream_t stream);
-void profile_after(int kind, hipStream_t stream);
-struct ProfileScope {
-  int kind;
-  hipStream_t stream;
-  ProfileScope(int k, hipStream_t s) : kind(k), stream(s) { profile_before(kind, stream); }
-  ~ProfileScope() { profile_after(kind, stream); }
-};
+// Per-kernel timing (gn_api.hip).  When profiling is enabled on this thread, profile_events hands out a
+// start / stop event pair that the launch binds to the kernel's own dispatch: their difference is the
+// kernel's begin-to-end time on the device, the quantity a kernel trace reports, with no dispatch gap.
+bool profile_events(int kind, hipEvent_t *start, hipEvent_t *stop);
+
+template <typename... KArgs, typename... Args>
+inline void launch(int kind, void (*kernel)(KArgs...), dim3 grid, dim3 block, hipStream_t stream, Args &&...args) {
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  if (profile_events(kind, &e0, &e1))
+    hipExtLaunchKernelGGL(kernel, grid, block, 0, stream, e0, e1, 0, static_cast<KArgs>(args)...);
+  else
+    hipLaunchKernelGGL(kernel, grid, block, 0, stream, static_cast<KArgs>(args)...);
+}
 
 // Return hipSuccess or the first launch error.
 template <typename T> hipError_t launch_fwd(const FwdArgs &a);

@@ -42,8 +42,8 @@ dim3 tile_grid(const Plan &p, int extra_x) {
 
 template <typename PT, int VEC, int ACT> void launch_apply(const FwdArgs &a, const A *part, const PartialGeo &q) {
   const Plan &p = a.plan;
-  hipLaunchKernelGGL((apply_kernel<elem_t, PT, VEC, ACT>), tile_grid(p, 0), dim3(kBlock), 0, a.stream, (const elem_t *)a.x,
-                     (elem_t *)a.y, part, q, a.w, a.b, a.mean, a.rstd, a.sdtype, (A)a.eps, p);
+  launch(kKindFwdApply, (apply_kernel<elem_t, PT, VEC, ACT>), tile_grid(p, 0), dim3(kBlock), a.stream, (const elem_t *)a.x,
+         (elem_t *)a.y, part, q, a.w, a.b, a.mean, a.rstd, a.sdtype, (A)a.eps, p);
 }
 template <typename PT, int VEC> void launch_apply_act(const FwdArgs &a, const A *part, const PartialGeo &q) {
   switch (a.act) {
@@ -147,8 +147,7 @@ template <typename PT, int ACT, int NV> bool try_resident_fwd_nv(const FwdArgs &
   if (!resident_tiling(a.plan, NV, slots, p)) return false;
   ResidentWorkspace r = resident_fwd_ws(a.ws, p);
   arm_generation(r, a.stream);
-  ProfileScope s(kKindFusedFwd, a.stream);
-  hipLaunchKernelGGL(kernel, tile_grid(p, 0), dim3(kBlock), 0, a.stream, (const elem_t *)a.x, (elem_t *)a.y, r.sync, a.w, a.b,
+  launch(kKindFusedFwd, kernel, tile_grid(p, 0), dim3(kBlock), a.stream, (const elem_t *)a.x, (elem_t *)a.y, r.sync, a.w, a.b,
                      a.mean, a.rstd, a.sdtype, (A)a.eps, p);
   return true;
 }
@@ -177,8 +176,7 @@ template <typename PT, int ACT, int NV> bool try_resident_bwd_nv(const BwdArgs &
   if (!resident_tiling(a.plan, NV, slots, p)) return false;
   ResidentWorkspace r = resident_bwd_ws(a.ws, p);
   arm_generation(r, a.stream);
-  ProfileScope s(kKindFusedBwd, a.stream);
-  hipLaunchKernelGGL(kernel, tile_grid(p, 0), dim3(kBlock), 0, a.stream, (const elem_t *)a.x, (const elem_t *)a.dy,
+  launch(kKindFusedBwd, kernel, tile_grid(p, 0), dim3(kBlock), a.stream, (const elem_t *)a.x, (const elem_t *)a.dy,
                      (elem_t *)a.dx, a.mean, a.rstd, a.sdtype, a.w, a.b, r.partC, r.sync, a.dw, a.db, p);
   return true;
 }
@@ -208,20 +206,17 @@ template <int VEC> hipError_t fwd_impl(const FwdArgs &a) {
   A *part = base + ws.part, *compact = base + ws.compact;
   PartialGeo q = {p.tiles, p.nchunk, p.lpr * p.vec};
   {
-    ProfileScope s(kKindFwdStats, a.stream);
-    hipLaunchKernelGGL((stats_kernel<elem_t, VEC>), tile_grid(p, 0), dim3(kBlock), 0, a.stream, (const elem_t *)a.x, part, p);
+    launch(kKindFwdStats, (stats_kernel<elem_t, VEC>), tile_grid(p, 0), dim3(kBlock), a.stream, (const elem_t *)a.x, part, p);
   }
   const A *src = part;
   if (needs_compaction(p)) {
-    ProfileScope s(kKindFwdStatsCompact, a.stream);
     const int64_t items = p.N * p.G;
     const unsigned grid = (unsigned)((items + kBlock / 64 - 1) / (kBlock / 64));
-    hipLaunchKernelGGL((stats_compact_kernel<A>), dim3(grid), dim3(kBlock), 0, a.stream, (const A *)part, compact, q, p);
+    launch(kKindFwdStatsCompact, (stats_compact_kernel<A>), dim3(grid), dim3(kBlock), a.stream, (const A *)part, compact, q, p);
     q = PartialGeo{1, 1, (int)p.C};
     src = compact;
   }
   {
-    ProfileScope s(kKindFwdApply, a.stream);
     if (a.pdtype == GN_INST_DTYPE) launch_apply_act<elem_t, VEC>(a, src, q);
     else launch_apply_act<wide_param_t, VEC>(a, src, q);
   }
@@ -235,24 +230,21 @@ template <typename PT, int VEC, int ACT> void launch_bwd_act(const BwdArgs &a) {
   A *partC = base + ws.partC, *partG = base + ws.partG, *compactC = base + ws.compactC, *compactG = base + ws.compactG;
   PartialGeo q = {p.tiles, p.nchunk, p.lpr * p.vec};
   {
-    ProfileScope s(kKindBwdReduce, a.stream);
-    hipLaunchKernelGGL((bwd_reduce_kernel<elem_t, PT, VEC, ACT>), tile_grid(p, 0), dim3(kBlock), 0, a.stream,
+    launch(kKindBwdReduce, (bwd_reduce_kernel<elem_t, PT, VEC, ACT>), tile_grid(p, 0), dim3(kBlock), a.stream,
                        (const elem_t *)a.x, (const elem_t *)a.dy, a.mean, a.rstd, a.sdtype, a.w, a.b, partC, partG, p);
   }
   const A *srcC = partC, *srcG = partG;
   if (needs_compaction(p)) {
-    ProfileScope s(kKindBwdCompact, a.stream);
     const int nG = (int)((p.N * p.G + kBlock / 64 - 1) / (kBlock / 64));
     const int64_t nC = (p.N * p.C + 31) / 32;
-    hipLaunchKernelGGL((bwd_compact_kernel<A>), dim3((unsigned)(nG + nC)), dim3(kBlock), 0, a.stream, (const A *)partC,
-                       (const A *)partG, compactC, compactG, q, nG, p);
+    launch(kKindBwdCompact, (bwd_compact_kernel<A>), dim3((unsigned)(nG + nC)), dim3(kBlock), a.stream, (const A *)partC,
+           (const A *)partG, compactC, compactG, q, nG, p);
     q = PartialGeo{1, 1, (int)p.C};
     srcC = compactC;
     srcG = compactG;
   }
   {
-    ProfileScope s(kKindBwdDx, a.stream);
-    hipLaunchKernelGGL((bwd_dx_kernel<elem_t, PT, VEC, ACT>), tile_grid(p, 1), dim3(kBlock), 0, a.stream,
+    launch(kKindBwdDx, (bwd_dx_kernel<elem_t, PT, VEC, ACT>), tile_grid(p, 1), dim3(kBlock), a.stream,
                        (const elem_t *)a.x, (const elem_t *)a.dy, (elem_t *)a.dx, a.mean, a.rstd, a.sdtype, a.w, a.b, srcC,
                        srcG, q, a.dw, a.db, p);
   }

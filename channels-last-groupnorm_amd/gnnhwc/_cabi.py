@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(_CSRC, "libgnnhwc_hip.so")
 
 # dtype / activation codes of include/gnnhwc.h
 F32, F64, F16, BF16 = 0, 1, 2, 3
-NUM_KERNEL_KINDS = 8
+NUM_KERNEL_KINDS = 9
 
 SYMBOLS = (
     "gnnhwc_version",
@@ -58,6 +58,8 @@ def _load():
     lib.gnnhwc_set_resident.restype = ci
     lib.gnnhwc_debug_read_trace.argtypes = [vp, i64]
     lib.gnnhwc_debug_read_trace.restype = ci
+    lib.gnnhwc_debug_copy.argtypes = [vp, vp, sz, vp]
+    lib.gnnhwc_debug_copy.restype = ci
     lib.gnnhwc_kernel_kind_name.argtypes = [ci]
     lib.gnnhwc_kernel_kind_name.restype = ctypes.c_char_p
     return lib

@@ -116,17 +116,27 @@ int gnnhwc_set_resident(int on);
 
 /*
  * Per-kernel timing for benchmarks (no counterpart in the reference, which relies on an external
- * profiler, prof.py:1-39).  While enabled, every kernel the library launches on this thread is
- * bracketed by HIP events on the launch stream.  gnnhwc_profile_collect synchronises those events and
+ * profiler, prof.py:1-39).  While enabled, every kernel the library launches on this thread carries a
+ * pair of HIP events bound to its own dispatch on the launch stream, so that their difference is the
+ * kernel's begin-to-end time on the device.  gnnhwc_profile_collect synchronises those events and
  * reports, for each kernel kind, the number of launches and the summed duration in milliseconds since
- * the last collect, then clears the record.  Kinds: 0 fwd statistics, 1 fwd statistics finalize,
- * 2 fwd apply, 3 bwd reduce, 4 bwd finalize, 5 bwd dx, 6 fused single-kernel fwd, 7 fused single-kernel bwd.
+ * the last collect, then clears the record.  Kinds: 0 fwd statistics, 1 fwd statistics compaction
+ * (many row tiles only), 2 fwd apply, 3 bwd reduce, 4 bwd compaction (many row tiles only), 5 bwd dx,
+ * 6 single-launch fwd, 7 single-launch bwd, 8 the plain copy of gnnhwc_debug_copy.
  */
-#define GNNHWC_NUM_KERNEL_KINDS 8
+#define GNNHWC_NUM_KERNEL_KINDS 9
 int gnnhwc_profile_enable(int on);
 int gnnhwc_profile_collect(int64_t *launches /* [GNNHWC_NUM_KERNEL_KINDS] */,
                            double *total_ms /* [GNNHWC_NUM_KERNEL_KINDS] */);
 const char *gnnhwc_kernel_kind_name(int kind);
+
+/*
+ * Plain device-to-device copy of `bytes` (a multiple of 16; 16-byte aligned pointers) by a kernel with the
+ * same block size and access width as the GroupNorm kernels and no arithmetic.  No counterpart in the
+ * reference.  Benchmarks use it as the practical ceiling a two-stream kernel can reach at a given size, and
+ * as the dispatch of known size that calibrates hardware memory-traffic counters.
+ */
+int gnnhwc_debug_copy(void *dst, const void *src, size_t bytes, void *stream /* hipStream_t */);
 
 /*
  * In-kernel timeline of the single-launch kernels, for tuning (no counterpart in the reference; its
