@@ -154,13 +154,17 @@ __device__ __forceinline__ void publish_tile(const SyncArea &s, int64_t idx) {
   }
 }
 
-// Wait until the `count` flags starting at `first` all carry this call's epoch.
-__device__ __forceinline__ void wait_flags(const SyncArea &s, int64_t first, int count) {
+// Wait until every (sample, row tile) workgroup of channel chunk k has raised its flag.
+__device__ __forceinline__ void wait_chunk_flags(const SyncArea &s, const Plan &p, int k) {
+  const int pairs = (int)p.N * p.tiles;
   int spins = 0;
   while (true) {
     int ok = 1;
-    for (int e = threadIdx.x; e < count; e += kBlock)
-      ok &= __hip_atomic_load(&s.flags[first + e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == s.epoch;
+    for (int e = threadIdx.x; e < pairs; e += kBlock) {
+      const int64_t nn = e / p.tiles;
+      const int t = e - (int)nn * p.tiles;
+      ok &= __hip_atomic_load(&s.flags[flag_index(p, nn, k, t)], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == s.epoch;
+    }
     if (__syncthreads_and(ok)) break;
     if (++spins > kMaxSpins) {
       if (threadIdx.x == 0) *s.status = s.epoch;
@@ -350,7 +354,11 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
           const A g = keep * vd[j] * act_bwd<ACT, A>(vx[j] * sa[j] + sb[j]);
           s1[j] += g * vx[j];
           s2[j] += g;
+          vd[j] = g;
         }
+        // dy is not needed again: its registers keep g' = dy * act'(z) for the dx phase (for 16-bit data
+        // rounded to T, the rounding an unfused activation backward applies to the same quantity)
+        bd[u] = LV::pack(vd);
       }
     }
     block_channel_sums<A, VEC>(p, l, s1, s2, sm1, sm2);
@@ -430,53 +438,49 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
       if (u < rows) {
         A vx[VEC], vd[VEC];
         pin(bx[u]);
-        pin(bd[u]);
         LV::unpack(bx[u], vx);
-        LV::unpack(bd[u], vd);
+        LV::unpack(bd[u], vd);  // g'
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) {
-          const A g = vd[j] * act_bwd<ACT, A>(vx[j] * sa[j] + sb[j]);
-          vd[j] = sa[j] * g + (c1[j] * vx[j] + c2[j]);
-        }
+        for (int j = 0; j < VEC; ++j) vd[j] = sa[j] * vd[j] + (c1[j] * vx[j] + c2[j]);
         LV::store(dx + off + (int64_t)u * step, LV::pack(vd));
       }
     }
   }
   trace_point(sync, 4);
-  // dgamma / dbeta for the channels of this chunk: row tile 0 of sample 0, once every sample's tiles of
-  // this chunk have published (compute_dweight_dbias, gn_kernel.cu:695-728)
-  if (l.tile == 0 && n == 0 && (dw || db)) {
-    for (int64_t nn = 0; nn < p.N; ++nn) wait_flags(sync, flag_index(p, nn, l.chunk, 0), p.tiles);
-    __syncthreads();
-    const int cw = l.wch < kBlock ? l.wch : kBlock;
-    const int nsl = kBlock / cw;
-    const int cl = threadIdx.x % cw, ts = threadIdx.x / cw;
-    for (int cbase = 0; cbase < l.wch; cbase += cw) {
-      const int c = l.cstart + cbase + cl;
-      A t1 = (A)0, t2 = (A)0;
-      if (cbase + cl < l.wch && ts < nsl) {
-        const int g = c / p.D;
-        for (int64_t nn = 0; nn < p.N; ++nn) {
-          A s1 = (A)0, s2 = (A)0;
-          for (int t = ts; t < p.tiles; t += nsl) {
+  // dgamma / dbeta (compute_dweight_dbias, gn_kernel.cu:695-728): the workgroups of sample 0 share the
+  // channels of their chunk, a segment of L lanes per channel summing over every (sample, row tile) pair,
+  // once all those tiles have published their per-channel sums.  The dx stores above drain meanwhile.
+  if (n == 0 && (dw || db)) {
+    const int pairs = (int)p.N * p.tiles;
+    const int L = pow2_ceil_clamped(pairs, 64);
+    const int cpp = kBlock / L;  // channels per pass of the workgroup
+    const int slot = threadIdx.x / L, sl = threadIdx.x % L;
+    if (l.tile * cpp < l.wch) {
+      wait_chunk_flags(sync, p, l.chunk);
+      for (int cb = l.tile * cpp; cb < l.wch; cb += p.tiles * cpp) {
+        const int cc = cb + slot;
+        const bool valid = cc < l.wch;
+        const int c = l.cstart + cc;
+        A t1 = (A)0, t2 = (A)0;
+        if (valid) {
+          const int g = c / p.D;
+          for (int e = sl; e < pairs; e += L) {
+            const int64_t nn = e / p.tiles;
+            const int t = e - (int)nn * p.tiles;
             const int64_t idx = ((nn * p.tiles + t) * p.C + c) * 2;
-            s1 += ld_part<true>(partC + idx);
-            s2 += ld_part<true>(partC + idx + 1);
+            const A s1 = ld_part<true>(partC + idx);
+            const A s2 = ld_part<true>(partC + idx + 1);
+            const A mu = load_scalar<A>(mean, nn * p.G + g, sdtype);
+            const A rs = load_scalar<A>(rstd, nn * p.G + g, sdtype);
+            t1 += (s1 - mu * s2) * rs;
+            t2 += s2;
           }
-          const A mu = load_scalar<A>(mean, nn * p.G + g, sdtype);
-          const A rs = load_scalar<A>(rstd, nn * p.G + g, sdtype);
-          t1 += (s1 - mu * s2) * rs;
-          t2 += s2;
         }
-      }
-      __syncthreads();
-      if (ts < nsl) { sm1[ts * cw + cl] = t1; sm2[ts * cw + cl] = t2; }
-      __syncthreads();
-      if (ts == 0 && cbase + cl < l.wch) {
-        A r1 = (A)0, r2 = (A)0;
-        for (int s = 0; s < nsl; ++s) { r1 += sm1[s * cw + cl]; r2 += sm2[s * cw + cl]; }
-        if (dw) store_param<PT, A>(dw, c, r1);
-        if (db) store_param<PT, A>(db, c, r2);
+        segment_sum2(t1, t2, L);
+        if (valid && sl == 0) {
+          if (dw) store_param<PT, A>(dw, c, t1);
+          if (db) store_param<PT, A>(db, c, t2);
+        }
       }
     }
     trace_point(sync, 5);
