@@ -89,14 +89,25 @@ Plan make_plan(int64_t N, int64_t R, int64_t C, int64_t G, int vec, int streams)
   if (forced_steps > 0) {
     k = forced_steps;
   } else {
-    // few, tall tiles: about `target` workgroups in all, so that the consumers' merge of tile partials stays short
+    // few, tall tiles: about `target` workgroups in all (one resident wave of them), so that the consumers' merge
+    // of tile partials stays short -- and, where that still leaves every CU busy, few enough tiles per group for
+    // the consumers to merge them in their prologue instead of a compaction launch in between
     int64_t tiles_wanted = (target + N * p.nchunk - 1) / (N * p.nchunk);
+    if (forced_target == 0) {
+      const int chunk_channels = lpr * vec;
+      const int64_t groups_touched = (chunk_channels + p.D - 2) / p.D + 1;
+      const int lanes = merge_lanes_for((int)(groups_touched < G ? groups_touched : G));
+      const int64_t tiles_merged = lanes < 1 ? 0 : (int64_t)kEarly * lanes / ((p.D - 1) / chunk_channels + 2);
+      if (tiles_wanted > tiles_merged && tiles_merged * N * p.nchunk >= kTargetBlocks / 2) tiles_wanted = tiles_merged;
+    }
     if (tiles_wanted < 1) tiles_wanted = 1;
     k = (lane_rows + tiles_wanted - 1) / tiles_wanted;
     if (k < unroll) {
       k = units / kNumCU;  // small problem: keep every CU busy before making tiles taller
       if (k < 1) k = 1;
       if (k > unroll) k = unroll;
+    } else {
+      k = (k + unroll - 1) / unroll * unroll;  // whole batches: no load slot of the last batch is wasted
     }
   }
   if (k > lane_rows) k = lane_rows;

@@ -236,9 +236,11 @@ template <typename PT, int VEC, int ACT> void launch_bwd_act(const BwdArgs &a) {
   const A *srcC = partC, *srcG = partG;
   if (needs_compaction(p)) {
     const int nG = (int)((p.N * p.G + kBlock / 64 - 1) / (kBlock / 64));
-    const int64_t nC = (p.N * p.C + 31) / 32;
+    int cpb = 32;  // channels per workgroup: fewer when N C is small, so that about a CU's worth of workgroups exist
+    while (cpb > 2 && p.N * p.C / cpb < kNumCU) cpb >>= 1;
+    const int64_t nC = (p.N * p.C + cpb - 1) / cpb;
     launch(kKindBwdCompact, (bwd_compact_kernel<A>), dim3((unsigned)(nG + nC)), dim3(kBlock), a.stream, (const A *)partC,
-           (const A *)partG, compactC, compactG, q, nG, p);
+           (const A *)partG, compactC, compactG, q, nG, cpb, p);
     q = PartialGeo{1, 1, (int)p.C};
     srcC = compactC;
     srcG = compactG;

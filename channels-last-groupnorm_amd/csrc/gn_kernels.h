@@ -814,12 +814,12 @@ __device__ __forceinline__ void sum_group_partials(const A *__restrict__ partG, 
 // ---------------------------------------------------------------------------------------------
 // Optional backward pass 1b (many tiles per sample): sum the tile partials once.
 //   blocks [0, nG)      : one wavefront per (n, g)         -> outG 2 planes [N][G]
-//   blocks [nG, nG + nC): eight lanes per (n, c)           -> outC [N][C][2]   (height_reduce, gn_kernel.cu:648-693)
+//   blocks [nG, nG + nC): kBlock / cpb lanes per (n, c)    -> outC [N][C][2]   (height_reduce, gn_kernel.cu:648-693)
 // ---------------------------------------------------------------------------------------------
 template <typename A>
 __global__ __launch_bounds__(kBlock) void bwd_compact_kernel(const A *__restrict__ partC, const A *__restrict__ partG,
                                                              A *__restrict__ outC, A *__restrict__ outG, PartialGeo q,
-                                                             int nG_blocks, Plan p) {
+                                                             int nG_blocks, int cpb, Plan p) {
   if ((int)blockIdx.x < nG_blocks) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int64_t item = (int64_t)blockIdx.x * (kBlock / 64) + wave;
@@ -834,28 +834,47 @@ __global__ __launch_bounds__(kBlock) void bwd_compact_kernel(const A *__restrict
     }
     return;
   }
-  // channel sums: 32 channels per workgroup, 8 tile slices; consecutive lanes read consecutive channels
-  const int cl = threadIdx.x & 31, ts = threadIdx.x >> 5;
-  const int64_t nc = ((int64_t)blockIdx.x - nG_blocks) * 32 + cl;
-  __shared__ A red[2][8][32];
+  // channel sums: cpb channels per workgroup (a power of two chosen by the host so that a small N C still
+  // yields many workgroups), kBlock / cpb tile slices; consecutive lanes read consecutive channels
+  const int cl = threadIdx.x & (cpb - 1), ts = threadIdx.x / cpb;
+  const int slices = kBlock / cpb;
+  const int64_t nc = ((int64_t)blockIdx.x - nG_blocks) * cpb + cl;
+  __shared__ A red[2][kBlock];
   const bool valid = nc < p.N * p.C;
   A t1 = (A)0, t2 = (A)0;
   if (valid) {
     const int64_t n = nc / p.C, c = nc - n * p.C;
-    for (int t = ts; t < q.tiles; t += 8) {
-      const int64_t idx = ((n * q.tiles + t) * p.C + c) * 2;
-      t1 += partC[idx];
-      t2 += partC[idx + 1];
+    const A *src = partC + ((n * q.tiles) * p.C + c) * 2;
+    const int64_t tstride = p.C * 2;
+    int t = ts;
+    for (; t + 3 * slices < q.tiles; t += 4 * slices) {  // four independent loads in flight per lane
+      A a[4], b[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        a[u] = src[(int64_t)(t + u * slices) * tstride];
+        b[u] = src[(int64_t)(t + u * slices) * tstride + 1];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) { t1 += a[u]; t2 += b[u]; }
+    }
+    for (; t < q.tiles; t += slices) {
+      t1 += src[(int64_t)t * tstride];
+      t2 += src[(int64_t)t * tstride + 1];
     }
   }
-  red[0][ts][cl] = t1;
-  red[1][ts][cl] = t2;
+  red[0][threadIdx.x] = t1;
+  red[1][threadIdx.x] = t2;
   __syncthreads();
+  for (int h = slices >> 1; h > 0; h >>= 1) {
+    if (ts < h) {
+      red[0][threadIdx.x] += red[0][threadIdx.x + h * cpb];
+      red[1][threadIdx.x] += red[1][threadIdx.x + h * cpb];
+    }
+    __syncthreads();
+  }
   if (valid && ts == 0) {
-    A r1 = (A)0, r2 = (A)0;
-    for (int s = 0; s < 8; ++s) { r1 += red[0][s][cl]; r2 += red[1][s][cl]; }
-    outC[nc * 2] = r1;
-    outC[nc * 2 + 1] = r2;
+    outC[nc * 2] = red[0][cl];
+    outC[nc * 2 + 1] = red[1][cl];
   }
 }
 

@@ -14,7 +14,7 @@ constexpr int kBlock = 256;         // threads per workgroup (4 wavefronts)
 constexpr int kUnrollFwd = 4;       // independent row loads in flight per lane, one-input kernels
 constexpr int kUnrollBwd = 2;       // ... two-input kernels (x and dy)
 constexpr int kNumCU = 256;         // MI355X
-constexpr int kTargetBlocks = 512;  // aim for ~2 workgroups per CU when the tensor is large enough
+constexpr int kTargetBlocks = 768;  // ~3 workgroups per CU, what the streaming kernels' registers allow: one resident wave
 constexpr int kEarly = 4;            // tile partials a lane of a consumer workgroup fetches ahead of its data
 
 // One workgroup owns `tile_rows` consecutive rows of one sample and one chunk of `lpr` lane vectors
