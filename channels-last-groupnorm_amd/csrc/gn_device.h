@@ -169,6 +169,16 @@ __device__ __forceinline__ double erf_acc(double x) { return erf(x); }
 __device__ __forceinline__ float exp_acc(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
 __device__ __forceinline__ double exp_acc(double x) { return exp(x); }
 
+// sigmoid(2u) for u = sqrt(2/pi) (z + 0.044715 z^3), with the constants of the exponent folded
+__device__ __forceinline__ float sigmoid_2u(float z, float z2) {
+  constexpr float k1 = (float)(-2.0 * 0.79788456080286535588 * 1.44269504088896340736);
+  constexpr float k3 = (float)(-2.0 * 0.79788456080286535588 * 1.44269504088896340736 * 0.044715);
+  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(z * (z2 * k3 + k1)));
+}
+__device__ __forceinline__ double sigmoid_2u(double z, double z2) {
+  return sigmoid(2.0 * 0.79788456080286535588 * (z + 0.044715 * z2 * z));
+}
+
 template <int ACT, typename A> __device__ __forceinline__ A act_fwd(A z) {
   if constexpr (ACT == GN_ACT_IDENTITY) {
     return z;
@@ -180,8 +190,7 @@ template <int ACT, typename A> __device__ __forceinline__ A act_fwd(A z) {
     return (A)0.5 * z * ((A)1 + erf_acc(z * (A)0.70710678118654752440));
   } else {
     // 1 + tanh(u) == 2 sigmoid(2u): the same function without the cancellation at u << 0
-    const A u = (A)0.79788456080286535588 * (z + (A)0.044715 * z * z * z);
-    return z * sigmoid((A)2 * u);
+    return z * sigmoid_2u(z, z * z);
   }
 }
 template <int ACT, typename A> __device__ __forceinline__ A act_bwd(A z) {
@@ -198,11 +207,10 @@ template <int ACT, typename A> __device__ __forceinline__ A act_bwd(A z) {
     return cdf + z * pdf;
   } else {
     const A z2 = z * z;
-    const A u = (A)0.79788456080286535588 * (z + (A)0.044715 * z2 * z);
-    const A du = (A)0.79788456080286535588 * ((A)1 + (A)0.134145 * z2);
-    const A s = sigmoid((A)2 * u);  // (1 + tanh u) / 2
-    // d/dz [z s] = s + z * 2 s (1 - s) * du
-    return s + (A)2 * z * s * ((A)1 - s) * du;
+    const A s = sigmoid_2u(z, z2);  // (1 + tanh u) / 2
+    const A du2 = z2 * (A)(2.0 * 0.79788456080286535588 * 0.134145) + (A)(2.0 * 0.79788456080286535588);  // 2 du/dz
+    // d/dz [z s] = s + z * 2 s (1 - s) * du/dz
+    return (z * s * du2) * ((A)1 - s) + s;
   }
 }
 
