@@ -70,7 +70,7 @@ Plan make_plan(int64_t N, int64_t R, int64_t C, int64_t G, int vec, int streams)
   if (forced_lpr > 0 && forced_lpr <= kBlock && forced_lpr <= p.cv) {
     lpr = forced_lpr;
   } else if (vec > 1) {
-    static const int preferred[] = {8, 16, 32, 64, 128, 256};
+    static const int preferred[] = {8, 16, 32, 64, 128, 256, 4, 2};  // half and quarter lines only as a last resort
     for (int d : preferred)
       if (p.cv % d == 0) { lpr = d; break; }
   }

@@ -164,8 +164,26 @@ __device__ __forceinline__ float sigmoid(float x) {
   return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.44269504088896340736f));
 }
 __device__ __forceinline__ double sigmoid(double x) { return 1.0 / (1.0 + exp(-x)); }
-__device__ __forceinline__ float erf_acc(float x) { return erff(x); }
-__device__ __forceinline__ double erf_acc(double x) { return erf(x); }
+// Standard normal CDF Phi(z) = (1 + erf(z / sqrt 2)) / 2.  fp32: erfc(t / sqrt 2) = exp2(t P(t)) for t = min(|z|, 6),
+// P a degree-10 least-squares fit of log2(erfc(t / sqrt 2)) / t on [0, 6] (result: absolute error 8e-8, relative
+// error 4e-6, so the left tail of Phi keeps its relative accuracy); straight-line code, no branches.
+__device__ __forceinline__ float normal_cdf(float z) {
+  const float t = fminf(fabsf(z), 6.0f);
+  float p = 2.729510037e-09f;
+  p = p * t + -1.013394950e-07f;
+  p = p * t + 1.666771318e-06f;
+  p = p * t + -1.587480181e-05f;
+  p = p * t + 9.414357042e-05f;
+  p = p * t + -3.183018466e-04f;
+  p = p * t + 5.031143559e-05f;
+  p = p * t + 6.909817011e-03f;
+  p = p * t + -5.242731270e-02f;
+  p = p * t + -4.592229807e-01f;
+  p = p * t + -1.151104130e+00f;
+  const float h = 0.5f * __builtin_amdgcn_exp2f(t * p);  // Phi(-|z|)
+  return z < 0.0f ? h : 1.0f - h;
+}
+__device__ __forceinline__ double normal_cdf(double z) { return 0.5 * erfc(z * -0.70710678118654752440); }
 __device__ __forceinline__ float exp_acc(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
 __device__ __forceinline__ double exp_acc(double x) { return exp(x); }
 
@@ -187,7 +205,7 @@ template <int ACT, typename A> __device__ __forceinline__ A act_fwd(A z) {
   } else if constexpr (ACT == GN_ACT_SILU) {
     return z * sigmoid(z);
   } else if constexpr (ACT == GN_ACT_GELU) {
-    return (A)0.5 * z * ((A)1 + erf_acc(z * (A)0.70710678118654752440));
+    return z * normal_cdf(z);
   } else {
     // 1 + tanh(u) == 2 sigmoid(2u): the same function without the cancellation at u << 0
     return z * sigmoid_2u(z, z * z);
@@ -202,7 +220,7 @@ template <int ACT, typename A> __device__ __forceinline__ A act_bwd(A z) {
     const A s = sigmoid(z);
     return s * ((A)1 + z * ((A)1 - s));
   } else if constexpr (ACT == GN_ACT_GELU) {
-    const A cdf = (A)0.5 * ((A)1 + erf_acc(z * (A)0.70710678118654752440));
+    const A cdf = normal_cdf(z);
     const A pdf = exp_acc((A)-0.5 * z * z) * (A)0.39894228040143267794;
     return cdf + z * pdf;
   } else {
