@@ -252,6 +252,30 @@ unsigned long long *trace_buffer() {
   }();
   return buf;
 }
+// Host-pinned, device-visible word that a single-launch kernel sets when one of its bounded waits expires
+// (its workgroups were not all resident at once, so its output is wrong).  The next API call reports it.
+unsigned long long *resident_status() {
+  static unsigned long long *word = []() -> unsigned long long * {
+    // the first call may come while the thread is capturing a graph: allocation is legal there in relaxed mode
+    hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+    const bool swapped = hipThreadExchangeStreamCaptureMode(&mode) == hipSuccess;
+    void *h = nullptr;
+    if (hipHostMalloc(&h, 64, hipHostMallocPortable | hipHostMallocMapped) != hipSuccess) {
+      (void)hipGetLastError();
+      h = nullptr;
+    }
+    if (swapped) (void)hipThreadExchangeStreamCaptureMode(&mode);
+    if (h) memset(h, 0, 64);
+    return (unsigned long long *)h;
+  }();
+  return word;
+}
+std::atomic<bool> g_status_live{false};  // resident_status() has been handed to a kernel
+void mark_resident_launch() { g_status_live.store(true, std::memory_order_relaxed); }
+
+std::atomic<int> g_spin_limit{1 << 22};
+int resident_spin_limit() { return g_spin_limit.load(std::memory_order_relaxed); }
+
 std::atomic<int> g_resident{-1};  // -1: follow the environment
 bool resident_enabled() {
   static const int off = env_int("GNNHWC_DISABLE_RESIDENT", 0);
@@ -275,6 +299,20 @@ bool profile_events(int kind, hipEvent_t *start, hipEvent_t *stop) {
 }  // namespace gn
 
 using namespace gn;
+
+// A timed-out single-launch kernel leaves wrong output behind: say so on the next call (nothing is launched by
+// that call), and use the streaming kernels for the rest of the process.
+static int check_resident_health() {
+  if (!g_status_live.load(std::memory_order_relaxed)) return GNNHWC_OK;
+  volatile unsigned long long *w = resident_status();
+  if (!w || *w == 0) return GNNHWC_OK;
+  *w = 0;
+  g_resident.store(0, std::memory_order_relaxed);
+  return fail(GNNHWC_ERR_LAUNCH,
+              "an earlier single-launch GroupNorm kernel could not synchronise its workgroups (they were not all resident "
+              "at once, e.g. because another stream was using the device); the results of that call are invalid. "
+              "The multi-launch kernels are used from now on");
+}
 
 extern "C" {
 
@@ -303,6 +341,8 @@ int gnnhwc_fwd(const void *x, const void *weight, const void *bias, void *y, voi
   if (act < GN_ACT_IDENTITY || act > GN_ACT_GELU_TANH)
     return fail(GNNHWC_ERR_INVALID_ARGUMENT, "unknown activation code %d", act);
   if (N == 0 || R == 0) return GNNHWC_OK;  // nothing to normalise; mean / rstd of an empty slab are left untouched
+  rc = check_resident_health();
+  if (rc != GNNHWC_OK) return rc;
   if (!x || !y || !mean || !rstd) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "x, y, mean and rstd must not be null");
   const size_t need = gnnhwc_fwd_workspace_bytes(N, R, C, G, dtype);
   if (!workspace || !aligned16(workspace) || workspace_bytes < need)
@@ -345,6 +385,8 @@ int gnnhwc_bwd(const void *dy, const void *x, const void *weight, const void *bi
     if (e0 != hipSuccess) return fail(GNNHWC_ERR_LAUNCH, "backward launch failed: %s", hipGetErrorString(e0));
     return GNNHWC_OK;
   }
+  rc = check_resident_health();
+  if (rc != GNNHWC_OK) return rc;
   if (!dy || !x || !mean || !rstd || !dx)
     return fail(GNNHWC_ERR_INVALID_ARGUMENT, "dy, x, mean, rstd and dx must not be null");
   const size_t need = gnnhwc_bwd_workspace_bytes(N, R, C, G, dtype);
@@ -402,6 +444,11 @@ int gnnhwc_set_resident(int on) {
   const int before = resident_enabled() ? 1 : 0;
   g_resident.store(on ? 1 : 0, std::memory_order_relaxed);
   return before;
+}
+
+int gnnhwc_debug_set_spin_limit(int polls) {
+  if (polls < 0) polls = 1 << 22;
+  return g_spin_limit.exchange(polls, std::memory_order_relaxed);
 }
 
 int gnnhwc_debug_read_trace(unsigned long long *out, int64_t count) {

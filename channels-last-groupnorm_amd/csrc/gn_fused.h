@@ -29,7 +29,7 @@
 
 namespace gn {
 
-constexpr int kMaxSpins = 1 << 22;
+constexpr int kMaxSpins = 1 << 22;  // default bound on the polls of one wait (seconds of polling)
 constexpr int kRecFast = 4;
 constexpr int kMaxResidentBlocksDev = 4 * kNumCU;  // records a lane keeps in registers while polling
 
@@ -40,6 +40,7 @@ struct SyncArea {
   unsigned long long epoch;   // value that marks "written in this call"
   const unsigned long long *generation;  // optional device word folded into the epoch (see resident_epoch)
   unsigned long long *status; // set to the epoch if a wait of this call timed out
+  int max_spins;              // polls allowed per wait
   unsigned long long *trace;  // optional [workgroup][kTracePoints] timestamps (100 MHz wall clock), else null
 };
 constexpr int kTracePoints = 8;
@@ -127,7 +128,7 @@ __device__ __forceinline__ void for_group_records(const SyncArea &s, __amdgpu_bu
 #pragma unroll
       for (int i = 0; i < kRecFast; ++i) ok = ok && (!have[i] || record_ready(rec[i], s.epoch));
       if (ok) break;
-      if (++spins > kMaxSpins) {
+      if (++spins > s.max_spins) {
         *s.status = s.epoch;
         break;
       }
@@ -166,7 +167,7 @@ __device__ __forceinline__ void wait_chunk_flags(const SyncArea &s, const Plan &
       ok &= __hip_atomic_load(&s.flags[flag_index(p, nn, k, t)], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == s.epoch;
     }
     if (__syncthreads_and(ok)) break;
-    if (++spins > kMaxSpins) {
+    if (++spins > s.max_spins) {
       if (threadIdx.x == 0) *s.status = s.epoch;
       break;
     }

@@ -91,7 +91,7 @@ bool resident_tiling(const Plan &base, int nv, int slots, Plan &out) {
 struct ResidentWorkspace {
   A *partC;  // backward only
   SyncArea sync;
-  unsigned long long *generation;  // device word behind the status word
+  unsigned long long *generation;  // device word behind the records / flags
 };
 // True while `stream` is recording into a HIP graph.
 bool stream_is_capturing(hipStream_t stream) {
@@ -117,8 +117,9 @@ ResidentWorkspace resident_fwd_ws(void *ws, const Plan &p) {
   r.sync.recs = base;
   r.sync.rec_bytes = (unsigned)resident_rec_bytes(p.G);
   r.sync.flags = nullptr;
-  r.sync.status = (unsigned long long *)(base + align_up(resident_rec_bytes(p.G), 256));
-  r.generation = r.sync.status + 1;
+  r.sync.status = resident_status();
+  r.generation = (unsigned long long *)(base + align_up(resident_rec_bytes(p.G), 256));
+  r.sync.max_spins = resident_spin_limit();
   r.sync.epoch = next_epoch();
   r.sync.trace = trace_buffer();
   return r;
@@ -133,8 +134,9 @@ ResidentWorkspace resident_bwd_ws(void *ws, const Plan &p) {
   r.sync.rec_bytes = (unsigned)resident_rec_bytes(p.G);
   char *f = recs + align_up(resident_rec_bytes(p.G), 256);
   r.sync.flags = (unsigned long long *)f;
-  r.sync.status = (unsigned long long *)(f + (size_t)kMaxResidentBlocks * 8);
-  r.generation = r.sync.status + 1;
+  r.sync.status = resident_status();
+  r.generation = (unsigned long long *)(f + (size_t)kMaxResidentBlocks * 8);
+  r.sync.max_spins = resident_spin_limit();
   r.sync.epoch = next_epoch();
   r.sync.trace = trace_buffer();
   return r;
@@ -146,6 +148,8 @@ template <typename PT, int ACT, int NV> bool try_resident_fwd_nv(const FwdArgs &
   Plan p;
   if (!resident_tiling(a.plan, NV, slots, p)) return false;
   ResidentWorkspace r = resident_fwd_ws(a.ws, p);
+  if (!r.sync.status) return false;
+  mark_resident_launch();
   arm_generation(r, a.stream);
   launch(kKindFusedFwd, kernel, tile_grid(p, 0), dim3(kBlock), a.stream, (const elem_t *)a.x, (elem_t *)a.y, r.sync, a.w, a.b,
                      a.mean, a.rstd, a.sdtype, (A)a.eps, p);
@@ -175,6 +179,8 @@ template <typename PT, int ACT, int NV> bool try_resident_bwd_nv(const BwdArgs &
   Plan p;
   if (!resident_tiling(a.plan, NV, slots, p)) return false;
   ResidentWorkspace r = resident_bwd_ws(a.ws, p);
+  if (!r.sync.status) return false;
+  mark_resident_launch();
   arm_generation(r, a.stream);
   launch(kKindFusedBwd, kernel, tile_grid(p, 0), dim3(kBlock), a.stream, (const elem_t *)a.x, (const elem_t *)a.dy,
                      (elem_t *)a.dx, a.mean, a.rstd, a.sdtype, a.w, a.b, r.partC, r.sync, a.dw, a.db, p);

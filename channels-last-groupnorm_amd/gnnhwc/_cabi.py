@@ -58,6 +58,8 @@ def _load():
     lib.gnnhwc_set_resident.restype = ci
     lib.gnnhwc_debug_read_trace.argtypes = [vp, i64]
     lib.gnnhwc_debug_read_trace.restype = ci
+    lib.gnnhwc_debug_set_spin_limit.argtypes = [ci]
+    lib.gnnhwc_debug_set_spin_limit.restype = ci
     lib.gnnhwc_debug_copy.argtypes = [vp, vp, sz, vp]
     lib.gnnhwc_debug_copy.restype = ci
     lib.gnnhwc_kernel_kind_name.argtypes = [ci]

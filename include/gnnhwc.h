@@ -131,6 +131,16 @@ int gnnhwc_profile_collect(int64_t *launches /* [GNNHWC_NUM_KERNEL_KINDS] */,
 const char *gnnhwc_kernel_kind_name(int kind);
 
 /*
+ * Failure handling of the single-launch kernels (no counterpart in the reference).  Their workgroups wait for
+ * each other with a bounded number of polls; if a wait expires (the workgroups were not all resident at once)
+ * the kernel still ends normally, its output is invalid, and the NEXT gnnhwc_fwd / gnnhwc_bwd call on any
+ * thread returns GNNHWC_ERR_LAUNCH without launching anything and switches the process to the multi-launch
+ * kernels.  gnnhwc_debug_set_spin_limit sets the number of polls per wait (negative: the default, 2^22) and
+ * returns the previous value; tests use 0 to exercise this path without hanging anything.
+ */
+int gnnhwc_debug_set_spin_limit(int polls);
+
+/*
  * Plain device-to-device copy of `bytes` (a multiple of 16; 16-byte aligned pointers) by a kernel with the
  * same block size and access width as the GroupNorm kernels and no arithmetic.  No counterpart in the
  * reference.  Benchmarks use it as the practical ceiling a two-stream kernel can reach at a given size, and

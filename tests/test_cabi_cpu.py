@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol():
     names = _declared_functions()
     assert {"gnnhwc_fwd", "gnnhwc_bwd", "gnnhwc_fwd_workspace_bytes", "gnnhwc_bwd_workspace_bytes", "gnnhwc_last_error",
             "gnnhwc_version", "gnnhwc_profile_enable", "gnnhwc_profile_collect", "gnnhwc_kernel_kind_name",
-            "gnnhwc_debug_read_trace", "gnnhwc_set_resident", "gnnhwc_debug_copy"} <= set(names)
+            "gnnhwc_debug_read_trace", "gnnhwc_set_resident", "gnnhwc_debug_copy", "gnnhwc_debug_set_spin_limit"} <= set(names)
     lib = ctypes.CDLL(_cabi.LIB_PATH)
     for n in names:
         assert hasattr(lib, n), n

@@ -338,3 +338,37 @@ def test_empty_and_wrapped_batches(family, device):
     t = orc.fwd_bwd(orc.to_nrc(x), w.double().cpu().numpy(), b.double().cpu().numpy(), orc.to_nrc(dy), G, 1e-5, 0)
     assert err(orc.to_nrc(y), t["y"]) <= 1e-5 and err(orc.to_nrc(xr.grad), t["dx"]) <= 1e-5
     assert err(wr.grad, t["dw"]) <= 1e-5 and err(br.grad, t["db"]) <= 1e-5
+
+
+def test_single_launch_timeout_is_reported(device):
+    """A single-launch kernel whose workgroups cannot wait for each other (forced here from the host with a poll
+    limit of 0, so every kernel still ends normally) leaves invalid output; the next call must say so, and the
+    calls after it run on the multi-launch kernels with correct results."""
+    lib = _cabi.lib
+    gen = torch.Generator().manual_seed(11)
+    N, R, C, G = 1, 4096, 1280, 32  # hundreds of workgroups: some poll is bound to come before its record
+    x = (torch.randn((N, R, C), generator=gen) * 2 + 1).to(torch.bfloat16).to(device)
+    w = (torch.rand(C, generator=gen) + 0.5).to(torch.bfloat16).to(device)
+    b = (0.1 * torch.randn(C, generator=gen)).to(torch.bfloat16).to(device)
+    truth = orc.fwd_bwd(x.double().cpu().numpy(), w.double().cpu().numpy(), b.double().cpu().numpy(),
+                        np.zeros((N, R, C)), G, 1e-5, 2)
+    before = _cabi.set_resident(True)
+    prev = lib.gnnhwc_debug_set_spin_limit(0)
+    try:
+        cabi_fwd(x, w, b, G, 1e-5, 2)
+        torch.cuda.synchronize()
+    finally:
+        lib.gnnhwc_debug_set_spin_limit(prev)
+    try:
+        with pytest.raises(RuntimeError, match="could not synchronise"):
+            cabi_fwd(x, w, b, G, 1e-5, 2)
+        y, mean, rstd = cabi_fwd(x, w, b, G, 1e-5, 2)  # multi-launch kernels from here on
+        torch.cuda.synchronize()
+        assert err(mean, truth["mean"]) <= 1e-5 and err(rstd, truth["rstd"]) <= 1e-5
+        assert err(y, truth["y"]) <= 2.0 ** -7
+        _cabi.set_resident(True)  # an explicit request re-enables the single-launch kernels
+        y2, mean2, _ = cabi_fwd(x, w, b, G, 1e-5, 2)
+        torch.cuda.synchronize()
+        assert err(mean2, truth["mean"]) <= 1e-5 and err(y2, truth["y"]) <= 2.0 ** -7
+    finally:
+        _cabi.set_resident(before)
