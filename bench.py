@@ -45,6 +45,7 @@ def parse_args():
     ap.add_argument("--workload", default="sd_unet")
     ap.add_argument("--all", action="store_true", help="also time every other configuration (reported under 'shapes')")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-shapes", action="store_true", help="skip the per-shape warm / cold / copy-ceiling table")
     ap.add_argument("--graph", action="store_true", help="time the replay of a HIP graph of the K steps instead of eager launches")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
     ap.add_argument("--counter-workload", action="store_true",
@@ -66,9 +67,9 @@ class Problem:
         x, dy = nrc_view(inp["x"]), nrc_view(inp["dy"])
         self.N, self.R, self.C = x.shape
         self.G = cfg.G
-        from oracle.gn_oracle import ACT_CODES  # name -> code table only
+        from gnnhwc.custom_gn import ACTIVATION_CODES
 
-        self.act = ACT_CODES[cfg.act]
+        self.act = ACTIVATION_CODES[cfg.act]
         self.w, self.b = inp["w"], inp["b"]
         self.sets = []
         for i in range(nsets):
@@ -186,27 +187,27 @@ def measure_shape(prob_warm, prob_cold, steps, warmup, use_graph):
 
 
 def kernel_profile(probs, steps):
-    """{shape: {kind: mean us}} over `steps` eager steps of the whole workload, from HIP events recorded on the
-    launch stream around each launch (the shapes run interleaved, as in the timed region)."""
+    """{shape: {kind: mean us}}: `steps` back-to-back eager steps per shape with a HIP event pair bound to every
+    launch on the launch stream (begin-to-end time of each dispatch), collected once per shape."""
     import torch
     from gnnhwc import _cabi
 
     stream = torch.cuda.current_stream().cuda_stream
-    acc = {p.cfg.name: {} for p in probs}
+    out = {}
     torch.cuda.synchronize()
     _cabi.profile_enable(True)
     try:
-        for _ in range(steps):
-            for p in probs:
+        for p in probs:
+            for _ in range(steps):  # untimed pass: creates the event pool, so that the host keeps ahead of the GPU below
                 p.step(0, stream)
-                for kind, (n, ms) in _cabi.profile_collect().items():
-                    if n:
-                        a = acc[p.cfg.name].setdefault(kind, [0, 0.0])
-                        a[0] += n
-                        a[1] += ms
+            _cabi.profile_collect()
+            for _ in range(steps):
+                p.step(0, stream)
+            res = _cabi.profile_collect()
+            out[p.cfg.name] = {k: ms / n * 1e3 for k, (n, ms) in res.items() if n}
     finally:
         _cabi.profile_enable(False)
-    return {name: {k: v[1] / v[0] * 1e3 for k, v in kinds.items()} for name, kinds in acc.items()}
+    return out
 
 
 def copy_ceiling(nbytes, device, steps):
@@ -290,7 +291,31 @@ def cpu_baseline(cfg_names, seconds):
         per[name] = round(med * 1e6, 1)
         total_bytes += configs.algorithmic_bytes(cfg)
         total_time += med
+    # second leg: the C restatement of the reference algorithm (float accumulation, OpenMP over its (n, g) slabs),
+    # on float32 copies of the same tensors; its bytes are counted at float32 width
+    oc_bytes, oc_time, oc_per = 0.0, 0.0, {}
+    for name in cfg_names:
+        cfg = configs.CONFIGS[name]
+        inp = configs.make_inputs(cfg, "cpu")
+        x = orc.to_nrc(inp["x"]).astype("float32")
+        dy = orc.to_nrc(inp["dy"]).astype("float32")
+        w, b = inp["w"].float().numpy(), inp["b"].float().numpy()
+        act = orc.ACT_CODES[cfg.act]
+        ts = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            if cfg.passes == "fwd":
+                orc.fwd(x, w, b, cfg.G, 1e-5, act, dtype="float32")
+            else:
+                orc.fwd_bwd(x, w, b, dy, cfg.G, 1e-5, act, dtype="float32")
+            ts.append(time.perf_counter() - t0)
+        med = statistics.median(ts)
+        oc_per[name] = round(med * 1e6, 1)
+        oc_bytes += (2 if cfg.passes == "fwd" else 5) * x.nbytes
+        oc_time += med
     return {
+        "oracle_c_f32": {"value": round(oc_bytes / oc_time / 1e9, 3), "unit": "GB/s (float32 tensors)", "us_per_call": oc_per,
+                         "sample": "oracle/gn_oracle.c float path, median of 3 calls per shape"},
         "value": round(total_bytes / total_time / 1e9, 3),
         "unit": "GB/s",
         "cores": torch.get_num_threads(),
@@ -367,7 +392,7 @@ def main():
 
     # ---- per-shape table ----
     shapes = {}
-    names = list(configs.ALL_NAMES) if args.all else head_names
+    names = [] if args.no_shapes else list(configs.ALL_NAMES) if args.all else head_names
     for n in names:
         cfg = configs.CONFIGS[n]
         S = configs.tensor_bytes(cfg)
@@ -393,7 +418,8 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5),
-        "us_per_call": {p.cfg.name: shapes[p.cfg.name].get("warm_fwd_bwd_us", shapes[p.cfg.name].get("warm_fwd_us")) for p in probs},
+        "us_per_call": {p.cfg.name: shapes[p.cfg.name].get("warm_fwd_bwd_us", shapes[p.cfg.name].get("warm_fwd_us"))
+                        for p in probs if p.cfg.name in shapes},
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
