@@ -114,6 +114,7 @@ Plan make_plan(int64_t N, int64_t R, int64_t C, int64_t G, int vec, int streams)
   p.tile_rows = (int)(k * p.rpi);
   p.tiles = (int)((R + p.tile_rows - 1) / p.tile_rows);
   p.nblocks = N * p.tiles * p.nchunk;
+  set_divisors(p);
   {
     const int chunk_channels = p.lpr * vec;
     const int64_t g = (chunk_channels + p.D - 2) / p.D + 1;  // groups a window of chunk_channels can touch
@@ -241,6 +242,10 @@ unsigned long long next_epoch() {
   unsigned long long e = seed + 0x9E3779B97F4A7C15ull * (counter.fetch_add(1) + 1);
   return e ? e : 1ull;
 }
+bool trace_waits() {
+  static const bool w = env_int("GNNHWC_TRACE", 0) != 2;
+  return w;
+}
 unsigned long long *trace_buffer() {
   static unsigned long long *buf = []() -> unsigned long long * {
     if (env_int("GNNHWC_TRACE", 0) == 0) return nullptr;
@@ -273,6 +278,10 @@ unsigned long long *resident_status() {
 std::atomic<bool> g_status_live{false};  // resident_status() has been handed to a kernel
 void mark_resident_launch() { g_status_live.store(true, std::memory_order_relaxed); }
 
+int resident_min_rows() {
+  static const int v = env_int("GNNHWC_RESIDENT_MIN_ROWS", 0);
+  return v;
+}
 std::atomic<int> g_spin_limit{1 << 22};
 int resident_spin_limit() { return g_spin_limit.load(std::memory_order_relaxed); }
 

@@ -42,11 +42,16 @@ struct SyncArea {
   unsigned long long *status; // set to the epoch if a wait of this call timed out
   int max_spins;              // polls allowed per wait
   unsigned long long *trace;  // optional [workgroup][kTracePoints] timestamps (100 MHz wall clock), else null
+  int trace_wait;             // stamps wait for outstanding memory operations first
 };
 constexpr int kTracePoints = 8;
-__device__ __forceinline__ void trace_point(const SyncArea &s, int point) {
-  if (s.trace) __builtin_amdgcn_s_waitcnt(0);  // stamp a phase only once its memory operations have completed
-  if (s.trace && threadIdx.x == 0) {
+__device__ __forceinline__ void trace_point(const SyncArea &s, int point, float after = 0.f) {
+  if (!s.trace) return;
+  // either stamp a phase once its memory operations have completed, or (trace_wait == 0) leave the kernel's
+  // own overlap alone and only order the stamp behind the value `after`
+  if (s.trace_wait) __builtin_amdgcn_s_waitcnt(0);
+  asm volatile("" ::"v"(after));
+  if (threadIdx.x == 0) {
     const int64_t b = ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
     if (b < kMaxResidentBlocksDev) s.trace[b * kTracePoints + point] = wall_clock64();
   }
@@ -117,7 +122,7 @@ __device__ __forceinline__ void for_group_records(const SyncArea &s, __amdgpu_bu
     for (int i = 0; i < kRecFast; ++i) {
       const int e = e0 + i * L;
       have[i] = e < P;
-      kk[i] = have[i] ? e / q.tiles : 0;
+      kk[i] = have[i] ? div_by(e, q.by_tiles) : 0;
       tt[i] = have[i] ? e - kk[i] * q.tiles : 0;
       idx[i] = base + kk[i] * kstride + tt[i];
     }
@@ -162,7 +167,7 @@ __device__ __forceinline__ void wait_chunk_flags(const SyncArea &s, const Plan &
   while (true) {
     int ok = 1;
     for (int e = threadIdx.x; e < pairs; e += kBlock) {
-      const int64_t nn = e / p.tiles;
+      const int64_t nn = div_by(e, p.by_tiles);
       const int t = e - (int)nn * p.tiles;
       ok &= __hip_atomic_load(&s.flags[flag_index(p, nn, k, t)], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == s.epoch;
     }
@@ -191,7 +196,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 8 
   const SyncArea sync = resident_epoch(sync_arg);
   __shared__ A sm0[kBlock * VEC];
   __shared__ A sm1[kBlock * VEC];
-  const PartialGeo q = {p.tiles, p.nchunk, p.lpr * p.vec};
+  const PartialGeo q = producer_geo(p);
   const int64_t n = blockIdx.z;
   const LanePos l = lane_pos(p, n, false);
   const int rows = l.rows;
@@ -233,7 +238,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 8 
     }
   }
   const __amdgpu_buffer_rsrc_t rb = record_buffer(sync);
-  trace_point(sync, 1);
+  trace_point(sync, 1, (float)m2[0]);
   block_group_moments<A, VEC>(p, l, mean, m2, sm0, sm1, [&](int g, A cnt, A mu, A s2) {
     (void)cnt;  // the consumers recompute it from the geometry
     record_store(rb, group_slot(q, p.G, n, l.tile, l.chunk, g), mu, s2, sync.epoch);
@@ -243,8 +248,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 8 
     // merge the records of the chunk's groups (exact two-pass form, compute_stats_pt2's job:
     // src/gnnhwc/csrc/gn_kernel.cu:226-292); rstd = 1 / sqrt(M2 / n + eps)
     const int L = merge_lanes(q, p.D);
-    const int nseg = kBlock / L;
-    const int seg = threadIdx.x / L, sl = threadIdx.x % L;
+    const int nseg = kBlock >> __builtin_ctz(L);  // L is a power of two
+    const int seg = threadIdx.x >> __builtin_ctz(L), sl = threadIdx.x & (L - 1);
     const A total = (A)p.D * (A)p.R;  // elements of a group
     for (int base = 0; base < l.ng; base += nseg) {
       const int gi = base + seg;
@@ -316,7 +321,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
   __shared__ A sm2[kBlock * VEC];
   __shared__ A sm_mu[kBlock * VEC];
   __shared__ A sm_rs[kBlock * VEC];
-  const PartialGeo q = {p.tiles, p.nchunk, p.lpr * p.vec};
+  const PartialGeo q = producer_geo(p);
   const int64_t n = blockIdx.z;
   const LanePos l = lane_pos(p, n, false);
   const __amdgpu_buffer_rsrc_t rb = record_buffer(sync);
@@ -362,6 +367,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
         bd[u] = LV::pack(vd);
       }
     }
+    trace_point(sync, 6, (float)(s1[0] + s2[0]));
     block_channel_sums<A, VEC>(p, l, s1, s2, sm1, sm2);
   }
   for (int c = threadIdx.x; c < l.wch; c += kBlock) {
@@ -376,8 +382,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
   __syncthreads();
   {
     const int L = pow2_ceil_clamped(p.D < l.wch ? p.D : l.wch, 64);
-    const int nseg = kBlock / L;
-    const int seg = threadIdx.x / L, sl = threadIdx.x % L;
+    const int nseg = kBlock >> __builtin_ctz(L);  // L is a power of two
+    const int seg = threadIdx.x >> __builtin_ctz(L), sl = threadIdx.x & (L - 1);
     for (int base = 0; base < l.ng; base += nseg) {
       const int gi = base + seg;
       const int g = l.g_lo + gi;
@@ -390,13 +396,12 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
       if (valid && sl == 0) record_store(rb, group_slot(q, p.G, n, l.tile, l.chunk, g), ta, tb, sync.epoch);
     }
   }
-  if (dw || db) publish_tile(sync, flag_index(p, n, l.chunk, l.tile));  // partC is complete: for the dgamma / dbeta workgroups
-  else __syncthreads();
+  __syncthreads();
   trace_point(sync, 2);
   {
     const int L = merge_lanes(q, p.D);
-    const int nseg = kBlock / L;
-    const int seg = threadIdx.x / L, sl = threadIdx.x % L;
+    const int nseg = kBlock >> __builtin_ctz(L);  // L is a power of two
+    const int seg = threadIdx.x >> __builtin_ctz(L), sl = threadIdx.x & (L - 1);
     for (int base = 0; base < l.ng; base += nseg) {
       const int gi = base + seg;
       const bool valid = gi < l.ng;
@@ -417,11 +422,14 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
       }
     }
   }
-  __syncthreads();
+  // partC went out before the records; by now those stores have long been acknowledged, so raising this tile's
+  // flag for the dgamma / dbeta workgroups costs no wait here (the barrier also orders the LDS writes above)
+  if (dw || db) publish_tile(sync, flag_index(p, n, l.chunk, l.tile));
+  else __syncthreads();
   trace_point(sync, 3);
   if (rows > 0) {
     {
-      int gi = (l.cvi * VEC) / p.D;
+      int gi = div_by(l.cvi * VEC, p.by_D);
       int rem = l.cvi * VEC - gi * p.D;
       gi -= l.g_lo;
 #pragma unroll
@@ -454,8 +462,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
   if (n == 0 && (dw || db)) {
     const int pairs = (int)p.N * p.tiles;
     const int L = pow2_ceil_clamped(pairs, 64);
-    const int cpp = kBlock / L;  // channels per pass of the workgroup
-    const int slot = threadIdx.x / L, sl = threadIdx.x % L;
+    const int cpp = kBlock >> __builtin_ctz(L);  // channels per pass of the workgroup (L is a power of two)
+    const int slot = threadIdx.x >> __builtin_ctz(L), sl = threadIdx.x & (L - 1);
     if (l.tile * cpp < l.wch) {
       wait_chunk_flags(sync, p, l.chunk);
       for (int cb = l.tile * cpp; cb < l.wch; cb += p.tiles * cpp) {
@@ -464,9 +472,9 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
         const int c = l.cstart + cc;
         A t1 = (A)0, t2 = (A)0;
         if (valid) {
-          const int g = c / p.D;
+          const int g = div_by(c, p.by_D);
           for (int e = sl; e < pairs; e += L) {
-            const int64_t nn = e / p.tiles;
+            const int64_t nn = div_by(e, p.by_tiles);
             const int t = e - (int)nn * p.tiles;
             const int64_t idx = ((nn * p.tiles + t) * p.C + c) * 2;
             const A s1 = ld_part<true>(partC + idx);

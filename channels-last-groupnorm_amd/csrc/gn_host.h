@@ -78,11 +78,13 @@ unsigned long long next_epoch();
 bool resident_enabled();
 // Device buffer for in-kernel timestamps when GNNHWC_TRACE=1, else null.
 unsigned long long *trace_buffer();
+bool trace_waits();  // GNNHWC_TRACE=1: stamps wait for memory; GNNHWC_TRACE=2: they do not
 // Host-pinned word the single-launch kernels set on a timed-out wait (null if it cannot be allocated: then the
 // single-launch kernels are not used), and the note that a kernel has been given it.
 unsigned long long *resident_status();
 void mark_resident_launch();
 int resident_spin_limit();
+int resident_min_rows();  // tuning knob (environment): smallest rows-per-lane variant the single-launch path may pick
 
 // Consumers merge the tile partials of their own groups in their prologue when every lane has at most kEarly
 // entries to fetch; otherwise a compaction kernel runs in between and leaves one entry per group.

@@ -85,6 +85,7 @@ bool resident_tiling(const Plan &base, int nv, int slots, Plan &out) {
   out.tile_rows = (int)rows;
   out.tiles = (int)tiles;
   out.nblocks = columns * tiles;
+  set_divisors(out);
   return true;
 }
 
@@ -122,6 +123,7 @@ ResidentWorkspace resident_fwd_ws(void *ws, const Plan &p) {
   r.sync.max_spins = resident_spin_limit();
   r.sync.epoch = next_epoch();
   r.sync.trace = trace_buffer();
+  r.sync.trace_wait = trace_waits() ? 1 : 0;
   return r;
 }
 ResidentWorkspace resident_bwd_ws(void *ws, const Plan &p) {
@@ -139,10 +141,12 @@ ResidentWorkspace resident_bwd_ws(void *ws, const Plan &p) {
   r.sync.max_spins = resident_spin_limit();
   r.sync.epoch = next_epoch();
   r.sync.trace = trace_buffer();
+  r.sync.trace_wait = trace_waits() ? 1 : 0;
   return r;
 }
 
 template <typename PT, int ACT, int NV> bool try_resident_fwd_nv(const FwdArgs &a) {
+  if (NV < resident_min_rows()) return false;
   auto kernel = fused_fwd_kernel<elem_t, PT, kVec, ACT, NV>;
   static const int slots = resident_slots(kernel);
   Plan p;
@@ -174,6 +178,7 @@ bool try_resident_fwd(const FwdArgs &a) {
 }
 
 template <typename PT, int ACT, int NV> bool try_resident_bwd_nv(const BwdArgs &a) {
+  if (NV < resident_min_rows()) return false;
   auto kernel = fused_bwd_kernel<elem_t, PT, kVec, ACT, NV>;
   static const int slots = resident_slots(kernel);
   Plan p;
@@ -210,7 +215,7 @@ template <int VEC> hipError_t fwd_impl(const FwdArgs &a) {
   const FwdWorkspace ws = fwd_workspace(p);
   A *base = (A *)a.ws;
   A *part = base + ws.part, *compact = base + ws.compact;
-  PartialGeo q = {p.tiles, p.nchunk, p.lpr * p.vec};
+  PartialGeo q = producer_geo(p);
   {
     launch(kKindFwdStats, (stats_kernel<elem_t, VEC>), tile_grid(p, 0), dim3(kBlock), a.stream, (const elem_t *)a.x, part, p);
   }
@@ -219,7 +224,7 @@ template <int VEC> hipError_t fwd_impl(const FwdArgs &a) {
     const int64_t items = p.N * p.G;
     const unsigned grid = (unsigned)((items + kBlock / 64 - 1) / (kBlock / 64));
     launch(kKindFwdStatsCompact, (stats_compact_kernel<A>), dim3(grid), dim3(kBlock), a.stream, (const A *)part, compact, q, p);
-    q = PartialGeo{1, 1, (int)p.C};
+    q = compacted_geo(p);
     src = compact;
   }
   {
@@ -234,7 +239,7 @@ template <typename PT, int VEC, int ACT> void launch_bwd_act(const BwdArgs &a) {
   const BwdWorkspace ws = bwd_workspace(p);
   A *base = (A *)a.ws;
   A *partC = base + ws.partC, *partG = base + ws.partG, *compactC = base + ws.compactC, *compactG = base + ws.compactG;
-  PartialGeo q = {p.tiles, p.nchunk, p.lpr * p.vec};
+  PartialGeo q = producer_geo(p);
   {
     launch(kKindBwdReduce, (bwd_reduce_kernel<elem_t, PT, VEC, ACT>), tile_grid(p, 0), dim3(kBlock), a.stream,
                        (const elem_t *)a.x, (const elem_t *)a.dy, a.mean, a.rstd, a.sdtype, a.w, a.b, partC, partG, p);
@@ -247,7 +252,7 @@ template <typename PT, int VEC, int ACT> void launch_bwd_act(const BwdArgs &a) {
     const int64_t nC = (p.N * p.C + cpb - 1) / cpb;
     launch(kKindBwdCompact, (bwd_compact_kernel<A>), dim3((unsigned)(nG + nC)), dim3(kBlock), a.stream, (const A *)partC,
            (const A *)partG, compactC, compactG, q, nG, cpb, p);
-    q = PartialGeo{1, 1, (int)p.C};
+    q = compacted_geo(p);
     srcC = compactC;
     srcG = compactG;
   }

@@ -46,19 +46,19 @@ __device__ __forceinline__ LanePos lane_pos(const Plan &p, int64_t n, bool rever
   l.tile = t;
   l.chunk = blockIdx.y;
   const int tid = threadIdx.x;
-  l.ty = tid / p.lpr;
+  l.ty = div_by(tid, p.by_lpr);
   l.tx = tid - l.ty * p.lpr;
   l.cvi = l.chunk * p.lpr + l.tx;
   l.row0 = (int64_t)l.tile * p.tile_rows;
   const int64_t rem = p.R - l.row0;
   l.len = rem < p.tile_rows ? (int)rem : p.tile_rows;
-  l.rows_base = l.len / p.rpi;
+  l.rows_base = div_by(l.len, p.by_rpi);
   l.rows_rem = l.len - l.rows_base * p.rpi;
   l.cstart = l.chunk * p.lpr * p.vec;
   const int lanes_here = p.cv - l.chunk * p.lpr < p.lpr ? p.cv - l.chunk * p.lpr : p.lpr;
   l.wch = lanes_here * p.vec;
-  l.g_lo = l.cstart / p.D;
-  l.ng = (l.cstart + l.wch - 1) / p.D - l.g_lo + 1;
+  l.g_lo = div_by(l.cstart, p.by_D);
+  l.ng = div_by(l.cstart + l.wch - 1, p.by_D) - l.g_lo + 1;
   l.active = l.ty < p.rpi && l.cvi < p.cv;
   l.rows = l.active ? l.rows_base + (l.ty < l.rows_rem ? 1 : 0) : 0;
   return l;
@@ -96,7 +96,7 @@ __device__ __forceinline__ void double_buffered(int nb, ISSUE &&issue, CONSUME &
 }
 // Batches every active lane of the workgroup walks: the lane rows with the most rows set the count.
 template <int U> __device__ __forceinline__ int block_batches(const Plan &p, const LanePos &l) {
-  const int rows_blk = (l.len + p.rpi - 1) / p.rpi;
+  const int rows_blk = div_by(l.len + p.rpi - 1, p.by_rpi);
   return (rows_blk + U - 1) / U;
 }
 __device__ __forceinline__ int clamp_row(int idx, int rows) { return idx < rows ? idx : rows - 1; }
@@ -135,12 +135,12 @@ __device__ __forceinline__ int64_t group_plane(const PartialGeo &q, int G, int64
 }
 // Chunks [k_lo, k_lo + nk) of the producer hold pieces of group g.
 __device__ __forceinline__ void group_chunks(const PartialGeo &q, int D, int g, int &k_lo, int &nk) {
-  k_lo = (g * D) / q.chunk_channels;
-  nk = ((g + 1) * D - 1) / q.chunk_channels - k_lo + 1;
+  k_lo = div_by(g * D, q.by_chunk);
+  nk = div_by((g + 1) * D - 1, q.by_chunk) - k_lo + 1;
 }
 // Lanes per group for a consumer's looping merge of tile partials (general path).
 __device__ __forceinline__ int merge_lanes(const PartialGeo &q, int D) {
-  return pow2_ceil_clamped(q.tiles * ((D - 1) / q.chunk_channels + 2), 64);
+  return pow2_ceil_clamped(q.tiles * (div_by(D - 1, q.by_chunk) + 2), 64);
 }
 
 // Early fetch of tile partials: every group of the chunk gets `L` lanes in a single round, and each lane
@@ -157,8 +157,8 @@ __device__ __forceinline__ void fetch_partials(EarlyPartials<A, NF> &e, const A 
   int gp = 1;
   while (gp < p.gmax) gp <<= 1;
   e.L = kBlock / gp < 64 ? kBlock / gp : 64;
-  e.gi = threadIdx.x / e.L;
-  e.sl = threadIdx.x % e.L;
+  e.gi = threadIdx.x >> __builtin_ctz(e.L);  // L is a power of two
+  e.sl = threadIdx.x & (e.L - 1);
   e.valid = e.gi < l.ng;
   const int g = l.g_lo + e.gi;
   int k_lo = 0, nk = 1;
@@ -170,7 +170,7 @@ __device__ __forceinline__ void fetch_partials(EarlyPartials<A, NF> &e, const A 
   for (int i = 0; i < kEarly; ++i) {
     const int en = e.sl + i * e.L;
     const bool have = en < e.P;
-    const int k = have ? en / q.tiles : 0, t = have ? en - k * q.tiles : 0;
+    const int k = have ? div_by(en, q.by_tiles) : 0, t = have ? en - k * q.tiles : 0;
     const int64_t slot = base + k * kstride + t;
 #pragma unroll
     for (int f = 0; f < NF; ++f) e.v[i][f] = have ? ld_part<COH>(part + f * plane + slot) : (A)0;
@@ -293,97 +293,80 @@ __device__ __forceinline__ void lane_stats(const T *__restrict__ x, const Plan &
   double_buffered(nb, issue, consume);
 }
 
-// Rows of the tile owned by the lane rows of wavefront wv (64 / lpr lane rows per wavefront).
-__device__ __forceinline__ int wave_rows(const Plan &p, const LanePos &l, int wv) {
-  const int tpw = 64 / p.lpr;
-  int extra = l.rows_rem - wv * tpw;
-  extra = extra < 0 ? 0 : (extra > tpw ? tpw : extra);
-  return tpw * l.rows_base + extra;
+// Sum of col[0], col[stride], ... (n entries) with eight reads in flight: the loop is latency bound otherwise.
+template <typename A> __device__ __forceinline__ A column_sum(const A *col, int stride, int n) {
+  A t[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) t[i] = (A)0;
+  int r = 0;
+  for (; r + 8 <= n; r += 8) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) t[i] += col[(r + i) * stride];
+  }
+  for (; r < n; ++r) t[0] += col[r * stride];
+  return ((t[0] + t[1]) + (t[2] + t[3])) + ((t[4] + t[5]) + (t[6] + t[7]));
 }
 
 // Merge the per-lane moments of a workgroup into one (count, mean, M2) triple per group of the chunk and
 // hand each to emit(g, count, mean, M2) (called by one lane per group).
-// When the lanes of a row divide the wavefront (lpr | 64, the usual case) the lane rows of a wavefront are
-// first merged with butterfly shuffles (Chan's update, Welford.h:44-65), so LDS only carries one entry per
-// wavefront and channel; otherwise every lane row goes through LDS.  The entries of a group are then
-// merged with the exact two-pass form.
+// Chan's pairwise update (Welford.h:44-65) costs several operations per value and step; instead every
+// lane re-expresses its moments as plain sums about a pivot shared by its channel column (the mean of the
+// column's first lane row, so the pivot lies inside the data and nothing cancels),
+//   S1 = n (mean - K),   S2 = M2 + n (mean - K)^2,
+// which add across lane rows with one LDS read and one addition each; the channels of a group, whose pivots
+// differ, are then merged about the group's first pivot.
 template <typename A, int VEC, typename EMIT>
 __device__ __forceinline__ void block_group_moments(const Plan &p, const LanePos &l, const A (&mean)[VEC],
-                                                    const A (&m2)[VEC], A *sm_mean, A *sm_m2, EMIT &&emit) {
+                                                    const A (&m2)[VEC], A *sm_s1, A *sm_s2, EMIT &&emit) {
+  __shared__ A sm_k[kBlock * VEC];
   const int W = p.lpr * VEC;
-  const bool wave_path = (64 % p.lpr) == 0;
-  int nrow;  // LDS rows per channel after the first step
-  if (wave_path) {
-    A mw[VEC], qw[VEC];
+  const int col0 = l.tx * VEC;
+  if (l.active && l.ty == 0) {
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) { mw[j] = mean[j]; qw[j] = m2[j]; }
-    A cnt = (A)l.rows;
-    for (int off = p.lpr; off < 64; off <<= 1) {
-      const A ocnt = shfl_xor_acc(cnt, off, 64);
-      const A nn = cnt + ocnt;
-      const A f = nn > (A)0 ? ocnt * fast_rcp(nn) : (A)0;
+    for (int j = 0; j < VEC; ++j) sm_k[col0 + j] = mean[j];
+  }
+  __syncthreads();
+  if (l.active) {
+    const A cnt = (A)l.rows;
+    const int at = (l.ty * p.lpr + l.tx) * VEC;
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        const A om = shfl_xor_acc(mw[j], off, 64);
-        const A oq = shfl_xor_acc(qw[j], off, 64);
-        const A d = om - mw[j];
-        mw[j] += d * f;
-        qw[j] += oq + d * d * cnt * f;
-      }
-      cnt = nn;
+    for (int j = 0; j < VEC; ++j) {
+      const A d = mean[j] - sm_k[col0 + j];
+      const A t = cnt * d;
+      sm_s1[at + j] = t;
+      sm_s2[at + j] = m2[j] + t * d;
     }
-    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-    if (lane < p.lpr && l.cvi < p.cv) {
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        sm_mean[wv * W + lane * VEC + j] = mw[j];
-        sm_m2[wv * W + lane * VEC + j] = qw[j];
-      }
-    }
-    nrow = kBlock / 64;
-  } else {
-    if (l.active) {
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        sm_mean[l.ty * W + l.tx * VEC + j] = mean[j];
-        sm_m2[l.ty * W + l.tx * VEC + j] = m2[j];
-      }
-    }
-    nrow = l.len < p.rpi ? l.len : p.rpi;
+  }
+  __syncthreads();
+  for (int col = threadIdx.x; col < 2 * l.wch; col += kBlock) {
+    const bool second = col >= l.wch;
+    A *arr = second ? sm_s2 : sm_s1;
+    const int c = second ? col - l.wch : col;
+    arr[c] = column_sum(arr + c, W, p.rpi);  // replaces lane row 0 of the column (only this thread touches the column)
   }
   __syncthreads();
   const int nc_max = p.D < l.wch ? p.D : l.wch;
   const int L = pow2_ceil_clamped(nc_max, 16);  // lanes per group: a DPP row at most
-  const int nseg = kBlock / L;
-  const int seg = threadIdx.x / L, sl = threadIdx.x % L;
-  const int tpw = wave_path ? 64 / p.lpr : 1;
+  const int nseg = kBlock >> __builtin_ctz(L);  // L is a power of two
+  const int seg = threadIdx.x >> __builtin_ctz(L), sl = threadIdx.x & (L - 1);
+  const A nrows = (A)l.len;
   for (int base = 0; base < l.ng; base += nseg) {
     const int gi = base + seg;
     const int g = l.g_lo + gi;
     const bool valid = gi < l.ng;
     int ca = 0, cb = 0;
     if (valid) group_span(p, l, g, ca, cb);
-    // one pass about the pivot K = mean of the group's first entry
-    const A K = valid ? sm_mean[ca] : (A)0;
+    const A K = valid ? sm_k[ca] : (A)0;
     A s1 = (A)0, s2 = (A)0;
-    for (int c = ca + sl; c < cb; c += L)
-      for (int r = 0; r < nrow; ++r) {
-        int rows_r;
-        if (wave_path) {
-          int extra = l.rows_rem - r * tpw;
-          extra = extra < 0 ? 0 : (extra > tpw ? tpw : extra);
-          rows_r = tpw * l.rows_base + extra;
-        } else {
-          rows_r = l.rows_base + (r < l.rows_rem ? 1 : 0);
-        }
-        const A rc = (A)rows_r;
-        const A d = sm_mean[r * W + c] - K;
-        s1 += rc * d;
-        s2 += sm_m2[r * W + c] + rc * d * d;
-      }
+    for (int c = ca + sl; c < cb; c += L) {
+      const A dk = sm_k[c] - K;
+      const A a1 = sm_s1[c];
+      s1 += a1 + nrows * dk;
+      s2 += sm_s2[c] + dk * ((A)2 * a1 + nrows * dk);
+    }
     segment_sum2(s1, s2, L);
     if (valid && sl == 0) {
-      const A total = (A)(cb - ca) * (A)l.len;
+      const A total = (A)(cb - ca) * nrows;
       const A dm = s1 / total;
       emit(g, total, K + dm, s2 - s1 * dm);
     }
@@ -392,51 +375,25 @@ __device__ __forceinline__ void block_group_moments(const Plan &p, const LanePos
 }
 
 // Sum the per-lane (s1, s2) pairs of a workgroup over its lane rows: afterwards sm1[c], sm2[c] hold the
-// tile's sums for channel c of the chunk (c < wch).  Same two routes as block_group_moments.
+// tile's sums for channel c of the chunk (c < wch).
 template <typename A, int VEC>
 __device__ __forceinline__ void block_channel_sums(const Plan &p, const LanePos &l, const A (&s1)[VEC], const A (&s2)[VEC],
                                                    A *sm1, A *sm2) {
   const int W = p.lpr * VEC;
-  int nrow;
-  if ((64 % p.lpr) == 0) {
-    A a1[VEC], a2[VEC];
+  if (l.active) {
+    const int at = (l.ty * p.lpr + l.tx) * VEC;
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) { a1[j] = s1[j]; a2[j] = s2[j]; }
-    for (int off = p.lpr; off < 64; off <<= 1) {
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        a1[j] += shfl_xor_acc(a1[j], off, 64);
-        a2[j] += shfl_xor_acc(a2[j], off, 64);
-      }
+    for (int j = 0; j < VEC; ++j) {
+      sm1[at + j] = s1[j];
+      sm2[at + j] = s2[j];
     }
-    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-    if (lane < p.lpr && l.cvi < p.cv) {
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        sm1[wv * W + lane * VEC + j] = a1[j];
-        sm2[wv * W + lane * VEC + j] = a2[j];
-      }
-    }
-    nrow = kBlock / 64;
-  } else {
-    if (l.active) {
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        sm1[l.ty * W + l.tx * VEC + j] = s1[j];
-        sm2[l.ty * W + l.tx * VEC + j] = s2[j];
-      }
-    }
-    nrow = p.rpi;
   }
   __syncthreads();
-  for (int c = threadIdx.x; c < l.wch; c += kBlock) {
-    A t1 = (A)0, t2 = (A)0;
-    for (int r = 0; r < nrow; ++r) {
-      t1 += sm1[r * W + c];
-      t2 += sm2[r * W + c];
-    }
-    sm1[c] = t1;  // replaces row 0 of the column (only this thread touches the column)
-    sm2[c] = t2;
+  for (int col = threadIdx.x; col < 2 * l.wch; col += kBlock) {
+    const bool second = col >= l.wch;
+    A *arr = second ? sm2 : sm1;
+    const int c = second ? col - l.wch : col;
+    arr[c] = column_sum(arr + c, W, p.rpi);  // replaces lane row 0 of the column (only this thread touches the column)
   }
   __syncthreads();
 }
@@ -482,7 +439,7 @@ __device__ __forceinline__ Moments<A> merge_group_partials(const A *__restrict__
   const int64_t kstride = (int64_t)G * q.tiles;
   A nl = (A)0, kl = (A)0, s1 = (A)0, s2 = (A)0;
   for (int e = sl; e < P; e += L) {
-    const int k = e / q.tiles, t = e - k * q.tiles;
+    const int k = div_by(e, q.by_tiles), t = e - k * q.tiles;
     const int64_t slot = base + k * kstride + t;
     const A cn = ld_part<COH>(part + slot);
     const A mu = ld_part<COH>(part + plane + slot);
@@ -539,8 +496,8 @@ __device__ __forceinline__ void merge_chunk_stats(const A *__restrict__ part, co
                                                   const LanePos &l, A eps, A *sm_mu, A *sm_rs, void *mean_out,
                                                   void *rstd_out, int sdtype) {
   const int L = merge_lanes(q, p.D);
-  const int nseg = kBlock / L;
-  const int seg = threadIdx.x / L, sl = threadIdx.x % L;
+  const int nseg = kBlock >> __builtin_ctz(L);  // L is a power of two
+  const int seg = threadIdx.x >> __builtin_ctz(L), sl = threadIdx.x & (L - 1);
   const int64_t plane = group_plane(q, p.G, p.N);
   for (int base = 0; base < l.ng; base += nseg) {
     const int gi = base + seg;
@@ -598,7 +555,7 @@ __device__ __forceinline__ void lane_coeffs(const Plan &p, const LanePos &l, con
                                             const A *sm_c1, const A *sm_c2, A (&sa)[VEC], A (&sb)[VEC], A (&c1)[VEC],
                                             A (&c2)[VEC]) {
   const int c = l.cvi * VEC;
-  int gi = c / p.D;
+  int gi = div_by(c, p.by_D);
   int rem = c - gi * p.D;
   gi -= l.g_lo;
 #pragma unroll
@@ -767,8 +724,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
     __syncthreads();
     {
       const int L = pow2_ceil_clamped(p.D < l.wch ? p.D : l.wch, 64);
-      const int nseg = kBlock / L;
-      const int seg = threadIdx.x / L, sl = threadIdx.x % L;
+      const int nseg = kBlock >> __builtin_ctz(L);  // L is a power of two
+      const int seg = threadIdx.x >> __builtin_ctz(L), sl = threadIdx.x & (L - 1);
       for (int base = 0; base < l.ng; base += nseg) {
         const int gi = base + seg;
         const int g = l.g_lo + gi;
@@ -802,7 +759,7 @@ __device__ __forceinline__ void sum_group_partials(const A *__restrict__ partG, 
   ta = (A)0;
   tb = (A)0;
   for (int e = sl; e < P; e += L) {
-    const int k = e / q.tiles, t = e - k * q.tiles;
+    const int k = div_by(e, q.by_tiles), t = e - k * q.tiles;
     const int64_t slot = base + k * kstride + t;
     ta += ld_part<COH>(partG + slot);
     tb += ld_part<COH>(partG + plane + slot);
@@ -994,8 +951,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
       }
     } else {
       const int L = merge_lanes(q, p.D);
-      const int nseg = kBlock / L;
-      const int seg = threadIdx.x / L, sl = threadIdx.x % L;
+      const int nseg = kBlock >> __builtin_ctz(L);  // L is a power of two
+      const int seg = threadIdx.x >> __builtin_ctz(L), sl = threadIdx.x & (L - 1);
       for (int base = 0; base < l.ng; base += nseg) {
         const int gi = base + seg;
         const bool valid = gi < l.ng;

@@ -17,6 +17,26 @@ constexpr int kNumCU = 256;         // MI355X
 constexpr int kTargetBlocks = 768;  // ~3 workgroups per CU, what the streaming kernels' registers allow: one resident wave
 constexpr int kEarly = 4;            // tile partials a lane of a consumer workgroup fetches ahead of its data
 
+// Division by a launch constant without the integer-division sequence (a few dozen instructions on this
+// hardware, all of them latency in a workgroup's prologue): q = umulhi(n, magic) with
+// magic = floor(2^32 / d) + 1 is exact for 0 <= n with n d < 2^32.  The host fills `magic` only when the
+// largest dividend it will see satisfies that; magic == 0 selects the ordinary division.
+struct Divisor {
+  int d;
+  unsigned magic;
+};
+inline Divisor make_divisor(int64_t d, int64_t max_n) {
+  Divisor v;
+  v.d = (int)d;
+  v.magic = 0;
+  if (d > 1 && max_n >= 0 && max_n < ((int64_t)1 << 32) / d) v.magic = (unsigned)((((uint64_t)1) << 32) / (uint64_t)d + 1);
+  return v;
+}
+__device__ __forceinline__ int div_by(int n, const Divisor &v) {
+  if (v.magic) return (int)__umulhi((unsigned)n, v.magic);
+  return v.d == 1 ? n : n / v.d;
+}
+
 // One workgroup owns `tile_rows` consecutive rows of one sample and one chunk of `lpr` lane vectors
 // (lpr * vec channels) of every such row.  Inside the workgroup thread t handles lane vector
 // (t % lpr) of rows (t / lpr), (t / lpr) + rpi, ...: every lane keeps the same channels for the whole
@@ -34,14 +54,44 @@ struct Plan {
   int tiles;        // row tiles per sample = ceil(R / tile_rows)
   int gmax;         // most groups any chunk intersects
   int64_t nblocks;  // N * tiles * nchunk
+  Divisor by_lpr, by_rpi, by_D, by_tiles, by_chunk;  // lpr, rpi, D, tiles, lpr * vec (set_divisors)
 };
+// Fill the divisors from the other fields (again after any change of the tiling).
+inline void set_divisors(Plan &p) {
+  p.by_lpr = make_divisor(p.lpr, kBlock);
+  p.by_rpi = make_divisor(p.rpi, (int64_t)p.tile_rows + p.rpi);
+  p.by_D = make_divisor(p.D, 2 * p.C);
+  const int64_t wide = p.N > p.nchunk + 1 ? p.N : p.nchunk + 1;
+  p.by_tiles = make_divisor(p.tiles, wide * p.tiles);
+  p.by_chunk = make_divisor((int64_t)p.lpr * p.vec, p.C + p.D);
+}
 
 // Geometry of a buffer of per-tile partial results as the consumer sees it: either the producer's own
 // (tiles, nchunk), or (1, 1) after the compaction kernel has merged all tiles of a sample.
 struct PartialGeo {
   int tiles, nchunk;
   int chunk_channels;  // channels per chunk of the producer (lpr * vec); C when compacted
+  Divisor by_tiles, by_chunk;
 };
+// The producer's own geometry, and the one a compaction kernel leaves behind.
+__host__ __device__ inline PartialGeo producer_geo(const Plan &p) {
+  PartialGeo q;
+  q.tiles = p.tiles;
+  q.nchunk = p.nchunk;
+  q.chunk_channels = p.lpr * p.vec;
+  q.by_tiles = p.by_tiles;
+  q.by_chunk = p.by_chunk;
+  return q;
+}
+inline PartialGeo compacted_geo(const Plan &p) {
+  PartialGeo q;
+  q.tiles = 1;
+  q.nchunk = 1;
+  q.chunk_channels = (int)p.C;
+  q.by_tiles = make_divisor(1, 0);
+  q.by_chunk = make_divisor(p.C, p.C + p.D);
+  return q;
+}
 
 // A consumer workgroup merges the tile partials of all groups of its chunk in one round: merge_lanes lanes
 // per group, each fetching at most kEarly entries.  The host checks that this covers the plan and
