@@ -340,6 +340,9 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
   }
   A sa[VEC], sb[VEC], c1[VEC], c2[VEC];
   if (rows > 0) lane_params<A, PT, VEC>(l, w, b, sa, sb);
+  // gamma of the channel this thread handles when the tile's per-channel sums are published: fetched now, so that
+  // the load is not part of the serial section between the sums and the record exchange
+  const A gamma0 = (w && (int)threadIdx.x < l.wch) ? load_param<PT, A>(w, l.cstart + threadIdx.x) : (A)1;
   stage_chunk_stats<A>(mean, rstd, sdtype, p, l, sm_mu, sm_rs);
   __syncthreads();
   trace_point(sync, 1);
@@ -375,7 +378,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
     const int64_t idx = ((n * p.tiles + l.tile) * p.C + l.cstart + c) * 2;
     st_part<true>(partC + idx, t1);
     st_part<true>(partC + idx + 1, t2);
-    const A gamma = w ? load_param<PT, A>(w, l.cstart + c) : (A)1;
+    const A gamma = c == (int)threadIdx.x ? gamma0 : (w ? load_param<PT, A>(w, l.cstart + c) : (A)1);
     sm1[c] = gamma * t1;
     sm2[c] = gamma * t2;
   }

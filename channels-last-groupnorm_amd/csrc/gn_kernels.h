@@ -409,7 +409,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
   using A = acc_t<T>;
   __shared__ A sm_mean[kBlock * VEC];
   __shared__ A sm_m2[kBlock * VEC];
-  const PartialGeo q = {p.tiles, p.nchunk, p.lpr * p.vec};
+  const PartialGeo q = producer_geo(p);
   const int64_t plane = group_plane(q, p.G, p.N);
   for (int64_t n = blockIdx.z; n < p.N; n += gridDim.z) {
     const LanePos l = lane_pos(p, n, false);
@@ -665,7 +665,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
   __shared__ A sm2[kBlock * VEC];
   __shared__ A sm_mu[kBlock * VEC];
   __shared__ A sm_rs[kBlock * VEC];
-  const PartialGeo q = {p.tiles, p.nchunk, p.lpr * p.vec};
+  const PartialGeo q = producer_geo(p);
   const int64_t plane = group_plane(q, p.G, p.N);
   for (int64_t n = blockIdx.z; n < p.N; n += gridDim.z) {
     const LanePos l = lane_pos(p, n, false);
@@ -698,6 +698,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
         }
       }
     };
+    // gamma of the channel this thread publishes in the epilogue, fetched now: off the tile's serial tail
+    const A gamma0 = (w && (int)threadIdx.x < l.wch) ? load_param<PT, A>(w, l.cstart + threadIdx.x) : (A)1;
     stage_chunk_stats<A>(mean, rstd, sdtype, p, l, sm_mu, sm_rs);  // small loads first, then the bulk
     if (rows > 0) {
       lane_params<A, PT, VEC>(l, w, b, sa, sb);
@@ -717,7 +719,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
       const int64_t idx = ((n * p.tiles + l.tile) * p.C + l.cstart + c) * 2;
       partC[idx] = t1;
       partC[idx + 1] = t2;
-      const A gamma = w ? load_param<PT, A>(w, l.cstart + c) : (A)1;
+      const A gamma = c == (int)threadIdx.x ? gamma0 : (w ? load_param<PT, A>(w, l.cstart + c) : (A)1);
       sm1[c] = gamma * t1;
       sm2[c] = gamma * t2;
     }
