@@ -50,6 +50,10 @@ __device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
 // unpack / pack convert to and from the accumulation type.
 template <typename T, int VEC> struct LaneVec;
 
+// Keeps the memory operations written before it ahead of those written after it in the instruction stream
+// (the scheduler is otherwise free to issue independent loads in any order, and loads return in issue order).
+__device__ __forceinline__ void issue_order_fence() { asm volatile("" ::: "memory"); }
+
 // Makes a register value opaque to the optimiser.  A kernel that keeps packed rows in registers across
 // several passes unpacks them again in every pass; without this the unpacked copies of one pass are
 // kept alive for the next, which doubles or triples the registers a 16-bit tile needs.
@@ -140,6 +144,29 @@ template <typename ACC> __device__ __forceinline__ ACC load_scalar(const void *p
     case GN_F16: return (ACC)(float)((const _Float16 *)p)[i];
     default: return (ACC)bf16_bits_to_float((uint32_t)((const uint16_t *)p)[i] << 16);
   }
+}
+// The same read without control flow: the candidate loads of every width are all issued (from `safe`, any
+// readable 8-byte-aligned address, when the width does not apply) and the result is selected.  A load under a
+// branch makes the compiler drain every outstanding load at the join; this form can sit next to bulk loads.
+template <typename ACC> __device__ __forceinline__ ACC load_scalar_flat(const void *p, int64_t i, int dtype, const void *safe) {
+  const bool half = dtype == GN_F16 || dtype == GN_BF16;
+  const float *pf = dtype == GN_F32 ? (const float *)p + i : (const float *)safe;
+  const uint16_t *ph = half ? (const uint16_t *)p + i : (const uint16_t *)safe;
+  const float vf = *pf;
+  const uint16_t vh = *ph;
+  ACC r;
+  if constexpr (sizeof(ACC) == 8) {
+    const double *pd = dtype == GN_F64 ? (const double *)p + i : (const double *)safe;
+    r = (ACC)*pd;
+  } else {
+    r = (ACC)0;
+  }
+  const float h16 = (float)__builtin_bit_cast(_Float16, vh);
+  const float b16 = bf16_bits_to_float((uint32_t)vh << 16);
+  if (dtype == GN_F32) r = (ACC)vf;
+  if (dtype == GN_F16) r = (ACC)h16;
+  if (dtype == GN_BF16) r = (ACC)b16;
+  return r;
 }
 template <typename ACC> __device__ __forceinline__ void store_scalar(void *p, int64_t i, int dtype, ACC v) {
   switch (dtype) {

@@ -326,24 +326,34 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
   const LanePos l = lane_pos(p, n, false);
   const __amdgpu_buffer_rsrc_t rb = record_buffer(sync);
   const int rows = l.rows;
-  const int64_t off = (n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC;
+  const SafeLane sfl = safe_lane<VEC>(p, l, n);
+  const int64_t off = sfl.off;
   const int64_t step = (int64_t)p.rpi * p.C;
   typename LV::raw_t bx[NV], bd[NV];
   trace_point(sync, 0);
-  if (rows > 0) {
-#pragma unroll
-    for (int u = 0; u < NV; ++u) {
-      const int64_t o = off + (int64_t)clamp_row(u, rows) * step;
-      bx[u] = LV::load(x + o);
-      bd[u] = LV::load(dy + o);
-    }
-  }
+  // the small loads go first: loads return in order, so the statistics and parameters, which the first row's
+  // arithmetic needs, must not queue behind the whole tile.  Nothing here is under a branch (idle lanes read valid
+  // addresses too), so every later wait counts exactly the loads it needs.
+  const StagedStats<A> st = fetch_chunk_stats<A>(mean, rstd, sdtype, p, l, sm_mu, sm_rs, partC);
   A sa[VEC], sb[VEC], c1[VEC], c2[VEC];
-  if (rows > 0) lane_params<A, PT, VEC>(l, w, b, sa, sb);
+  lane_params_flat<A, PT, VEC>(sfl.c, w, b, partC, sa, sb);
   // gamma of the channel this thread handles when the tile's per-channel sums are published: fetched now, so that
   // the load is not part of the serial section between the sums and the record exchange
-  const A gamma0 = (w && (int)threadIdx.x < l.wch) ? load_param<PT, A>(w, l.cstart + threadIdx.x) : (A)1;
-  stage_chunk_stats<A>(mean, rstd, sdtype, p, l, sm_mu, sm_rs);
+  A gamma0;
+  {
+    const int cg = (int)threadIdx.x < l.wch ? threadIdx.x : 0;
+    const PT *gp = w ? (const PT *)w + l.cstart + cg : (const PT *)partC;
+    const A gv = load_param<PT, A>(gp, 0);
+    gamma0 = w ? gv : (A)1;
+  }
+  issue_order_fence();
+#pragma unroll
+  for (int u = 0; u < NV; ++u) {
+    const int64_t o = off + (int64_t)clamp_row(u, sfl.rows) * step;
+    bx[u] = LV::load(x + o);
+    bd[u] = LV::load(dy + o);
+  }
+  commit_chunk_stats<A>(st, l, sm_mu, sm_rs);
   __syncthreads();
   trace_point(sync, 1);
   {

@@ -516,13 +516,30 @@ __device__ __forceinline__ void merge_chunk_stats(const A *__restrict__ part, co
   }
   __syncthreads();
 }
-// Backward: the caller's mean / rstd of the chunk's groups, staged in LDS the same way.
+// Backward: the caller's mean / rstd of the chunk's groups, staged in LDS the same way.  In two steps, so that
+// the loads can be issued ahead of a kernel's bulk loads and waited for on their own while those are in flight:
+// fetch (no control flow around the loads of the usual case, one group per thread) and commit (LDS writes).
+template <typename A> struct StagedStats {
+  A mu, rs;
+};
 template <typename A>
-__device__ __forceinline__ void stage_chunk_stats(const void *mean, const void *rstd, int sdtype, const Plan &p,
-                                                  const LanePos &l, A *sm_mu, A *sm_rs) {
-  for (int gi = threadIdx.x; gi < l.ng; gi += kBlock) {
+__device__ __forceinline__ StagedStats<A> fetch_chunk_stats(const void *mean, const void *rstd, int sdtype, const Plan &p,
+                                                            const LanePos &l, A *sm_mu, A *sm_rs, const void *safe) {
+  for (int gi = threadIdx.x + kBlock; gi < l.ng; gi += kBlock) {  // more groups than threads: rare, done up front
     sm_mu[gi] = load_scalar<A>(mean, l.n * p.G + l.g_lo + gi, sdtype);
     sm_rs[gi] = load_scalar<A>(rstd, l.n * p.G + l.g_lo + gi, sdtype);
+  }
+  const int gi = (int)threadIdx.x < l.ng ? threadIdx.x : l.ng - 1;
+  StagedStats<A> st;
+  st.mu = load_scalar_flat<A>(mean, l.n * p.G + l.g_lo + gi, sdtype, safe);
+  st.rs = load_scalar_flat<A>(rstd, l.n * p.G + l.g_lo + gi, sdtype, safe);
+  return st;
+}
+template <typename A>
+__device__ __forceinline__ void commit_chunk_stats(const StagedStats<A> &st, const LanePos &l, A *sm_mu, A *sm_rs) {
+  if ((int)threadIdx.x < l.ng) {
+    sm_mu[threadIdx.x] = st.mu;
+    sm_rs[threadIdx.x] = st.rs;
   }
 }
 
@@ -546,6 +563,39 @@ __device__ __forceinline__ void lane_params(const LanePos &l, const void *w, con
 #pragma unroll
     for (int j = 0; j < VEC; ++j) beta[j] = (A)0;
   }
+}
+// The same without control flow, for kernels whose bulk loads are all issued up front: a load under a branch
+// makes the compiler drain every outstanding load where the branch joins.  Absent parameters are read from
+// `safe` (any readable 64 bytes) and replaced by 1 / 0; c is the lane's first channel, already clamped into range.
+template <typename A, typename PT, int VEC>
+__device__ __forceinline__ void lane_params_flat(int c, const void *w, const void *b, const void *safe, A (&gamma)[VEC],
+                                                 A (&beta)[VEC]) {
+  const PT *wp = w ? (const PT *)w + c : (const PT *)safe;
+  const PT *bp = b ? (const PT *)b + c : (const PT *)safe;
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    const A gv = load_param<PT, A>(wp, j);
+    const A bv = load_param<PT, A>(bp, j);
+    gamma[j] = w ? gv : (A)1;
+    beta[j] = b ? bv : (A)0;
+  }
+}
+// Addresses that are valid for every lane of the workgroup, idle ones included (they re-read the tile's first
+// row and the row's last lane vector), so that loads need no guard; `rows` is at least 1 for the row clamp.
+struct SafeLane {
+  int64_t off;  // element offset of the lane's first row
+  int c;        // first channel of the lane vector
+  int rows;     // max(rows of the lane, 1)
+  bool live;    // the lane owns at least one row
+};
+template <int VEC> __device__ __forceinline__ SafeLane safe_lane(const Plan &p, const LanePos &l, int64_t n) {
+  SafeLane s;
+  s.live = l.rows > 0;
+  const int cvi = l.cvi < p.cv ? l.cvi : p.cv - 1;
+  s.c = cvi * VEC;
+  s.off = (n * p.R + l.row0 + (s.live ? l.ty : 0)) * p.C + s.c;
+  s.rows = s.live ? l.rows : 1;
+  return s;
 }
 // a = rstd * gamma, b = beta - mean * a: normalise + affine as one FMA per element (same folding as
 // src/gnnhwc/csrc/gn_kernel.cu:350-379, 601-602, 783-784).  Group statistics come from LDS; optional
@@ -700,11 +750,13 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
     };
     // gamma of the channel this thread publishes in the epilogue, fetched now: off the tile's serial tail
     const A gamma0 = (w && (int)threadIdx.x < l.wch) ? load_param<PT, A>(w, l.cstart + threadIdx.x) : (A)1;
-    stage_chunk_stats<A>(mean, rstd, sdtype, p, l, sm_mu, sm_rs);  // small loads first, then the bulk
+    // small loads first, then the bulk; the statistics are waited for on their own
+    const StagedStats<A> st = fetch_chunk_stats<A>(mean, rstd, sdtype, p, l, sm_mu, sm_rs, partC);
     if (rows > 0) {
       lane_params<A, PT, VEC>(l, w, b, sa, sb);
       issue(std::integral_constant<int, 0>{}, 0);
     }
+    commit_chunk_stats<A>(st, l, sm_mu, sm_rs);
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < VEC; ++j) { s1[j] = (A)0; s2[j] = (A)0; }
