@@ -340,6 +340,53 @@ def test_empty_and_wrapped_batches(family, device):
     assert err(wr.grad, t["dw"]) <= 1e-5 and err(br.grad, t["db"]) <= 1e-5
 
 
+# The reference's own regression list (test/check_outputs.py:161-185: identity activation, float64) and a seeded
+# sample of its brute-force grid (test/check_outputs.py:191-211: bfloat16, H == W, batch sizes / channel counts /
+# resolutions / group counts from the same lists).
+REFERENCE_CUSTOM_INPUTS = [
+    (1, 1, 2, 2, 1), (2, 3909, 5, 5, 3), (1, 2062, 5, 5, 1031), (3, 4096, 7, 7, 4), (1, 4096, 7, 7, 4),
+    (2, 160, 8, 8, 160), (1, 3, 7, 7, 1), (1, 1, 4, 4, 1), (1, 128, 8, 8, 8), (2, 1280, 8, 8, 32),
+    (2, 640, 16, 16, 32), (2, 2560, 8, 8, 32), (2, 1280, 16, 16, 32), (2, 320, 32, 32, 32), (2, 1920, 16, 16, 32),
+    (2, 2560, 16, 16, 32), (2, 640, 32, 32, 32), (2, 960, 32, 32, 32), (2, 1280, 32, 32, 32), (2, 320, 64, 64, 32),
+    (2, 1920, 32, 32, 32), (2, 640, 64, 64, 32), (8, 128, 64, 64, 32),
+]
+
+
+@pytest.mark.parametrize("B,C,H,W,G", REFERENCE_CUSTOM_INPUTS)
+def test_reference_custom_inputs(B, C, H, W, G, device):
+    gen = torch.Generator().manual_seed(B * 7919 + C)
+    shape = (B, C, H, W)
+    x = channels_last_like(shape, torch.float64, device, gen, 1.3, 0.2)
+    dy = channels_last_like(shape, torch.float64, device, gen)
+    w = (torch.rand(C, generator=gen, dtype=torch.float64) + 0.5).to(device)
+    b = (0.1 * torch.randn(C, generator=gen, dtype=torch.float64)).to(device)
+    check_against_torch(x, G, "identity", w, b, dy)
+
+
+def _brute_force_sample(count, seed):
+    import itertools
+    import random
+
+    Bs = (1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 13, 16)
+    Cs = (1, 2, 3, 4, 5, 6, 7, 32, 64, 128, 256, 512, 13, 140, 125, 961, 160, 320, 640, 960, 1280, 1600, 1920, 2240, 2560,
+          1303, 2602, 3909)
+    Rs = (2, 3, 4, 5, 6, 7, 8, 9, 10, 17, 16, 64, 128)
+    Gs = (1, 2, 3, 4, 8, 16, 32)
+    valid = [(B, C, R, G) for B, C, R, G in itertools.product(Bs, Cs, Rs, Gs) if C % G == 0 and B * C * R * R <= (1 << 24)]
+    return random.Random(seed).sample(valid, count)
+
+
+@pytest.mark.parametrize("B,C,R,G", _brute_force_sample(48, 2024))
+def test_reference_brute_force_sample(family, B, C, R, G, device):
+    gen = torch.Generator().manual_seed(B * 31 + C * 7 + R)
+    shape = (B, C, R, R)
+    x = channels_last_like(shape, torch.bfloat16, device, gen, 1.0, 0.0)
+    dy = channels_last_like(shape, torch.bfloat16, device, gen)
+    w = (torch.rand(C, generator=gen) + 0.5).to(torch.bfloat16).to(device)
+    b = (0.1 * torch.randn(C, generator=gen)).to(torch.bfloat16).to(device)
+    check_against_torch(x, G, "identity", w, b, dy)
+
+
 def test_single_launch_timeout_is_reported(device):
     """A single-launch kernel whose workgroups cannot wait for each other (forced here from the host with a poll
     limit of 0, so every kernel still ends normally) leaves invalid output; the next call must say so, and the
