@@ -143,6 +143,27 @@ _op_lib.impl("fwd", gn_nhwc_fwd, "CompositeExplicitAutograd")
 _op_lib.impl("bwd", gn_nhwc_bwd, "CompositeExplicitAutograd")
 
 
+def _fwd_meta(X, weight, bias, G, eps, act_fn_option):
+    """Shapes, dtypes and strides of gnop::fwd's outputs for meta / fake tensors (tracing): Y keeps X's
+    (N, C, R) shape with strides (R*C, 1, C), as the permuted view returned by the real operator does."""
+    N, C, R = X.shape
+    Y = torch.empty((N, R, C), dtype=X.dtype, device=X.device).permute(0, 2, 1)
+    sdtype = _stats_dtype(X.dtype)
+    return Y, torch.empty((N, G), dtype=sdtype, device=X.device), torch.empty((N, G), dtype=sdtype, device=X.device)
+
+
+def _bwd_meta(dy, X, weight, bias, means, rstds, G, act_fn_option):
+    N, C, R = X.shape
+    dX = torch.empty((N, R, C), dtype=X.dtype, device=X.device).permute(0, 2, 1)
+    return dX, torch.empty((C,), dtype=weight.dtype, device=X.device), torch.empty((C,), dtype=weight.dtype, device=X.device)
+
+
+# The reference's operators cannot be traced (its forward is wrapped in torch._dynamo.disable, custom_gn.py:63);
+# with these the operators at least carry correct output metadata under fake-tensor tracing.
+_op_lib.impl("fwd", _fwd_meta, "Meta")
+_op_lib.impl("bwd", _bwd_meta, "Meta")
+
+
 class GN_NHWC_Func(torch.autograd.Function):
     """custom_gn.py:29-47.  apply(X, weight, bias, G, eps, activation_code) -> Y with X's shape and strides."""
 

@@ -125,3 +125,20 @@ def test_channels_first_input_takes_the_torch_fallback(act):
     assert x.grad is not None and m.weight.grad is not None
     m2 = GN_NHWC(4, 8, activation=act, affine=False)
     assert torch.allclose(m2(x), orc.torch_act(act)(torch.nn.functional.group_norm(x, 4, None, None, m2.eps)), rtol=1e-5, atol=1e-6)
+
+
+def test_operator_metadata_on_meta_tensors():
+    """gnop::fwd / gnop::bwd report the shapes, dtypes and channels-last strides of their outputs for meta tensors
+    (what fake-tensor tracing sees); no kernel runs."""
+    import torch
+    import gnnhwc  # noqa: F401  (registers the operators)
+
+    N, C, R, G = 3, 8, 20, 2
+    for dtype, sdtype in ((torch.float32, torch.float32), (torch.bfloat16, torch.float32), (torch.float64, torch.float64)):
+        X = torch.empty((N, R, C), dtype=dtype, device="meta").permute(0, 2, 1)
+        w = torch.empty((C,), dtype=dtype, device="meta")
+        Y, mean, rstd = torch.ops.gnop.fwd(X, w, w, G, 1e-5, 2)
+        assert Y.shape == (N, C, R) and Y.stride() == (R * C, 1, C) and Y.dtype == dtype
+        assert mean.shape == (N, G) and rstd.shape == (N, G) and mean.dtype == sdtype
+        dX, dw, db = torch.ops.gnop.bwd(X, X, w, w, mean, rstd, G, 2)
+        assert dX.shape == (N, C, R) and dX.stride() == (R * C, 1, C) and dw.shape == (C,) and db.dtype == dtype
