@@ -147,9 +147,10 @@ __device__ __forceinline__ int merge_lanes(const PartialGeo &q, int D) {
 // loads its (at most kEarly) entries of NF fields into registers.  The loads are issued before the lane's
 // first data loads, so they are not queued behind them; they are consumed after those loads are in flight.
 template <typename A, int NF> struct EarlyPartials {
-  A v[kEarly][NF];
+  A v[kEarly][NF];  // as loaded: entry i is meaningful only if have(i) (the others were read from entry 0 of the buffer)
   int L, gi, sl, P;
   bool valid;
+  __device__ __forceinline__ bool have(int i) const { return sl + i * L < P; }
 };
 template <typename A, int NF, bool COH>
 __device__ __forceinline__ void fetch_partials(EarlyPartials<A, NF> &e, const A *__restrict__ part, int64_t plane,
@@ -166,27 +167,34 @@ __device__ __forceinline__ void fetch_partials(EarlyPartials<A, NF> &e, const A 
   e.P = e.valid ? q.tiles * nk : 0;
   const int64_t base = group_slot(q, p.G, l.n, 0, k_lo, g);
   const int64_t kstride = (int64_t)p.G * q.tiles;
+  // all addresses first, then nothing but loads: any control flow between the loads (the division below may
+  // branch) or any use of a loaded value here would make the compiler wait for them before the caller's next loads
+  int64_t slot[kEarly];
 #pragma unroll
   for (int i = 0; i < kEarly; ++i) {
     const int en = e.sl + i * e.L;
     const bool have = en < e.P;
     const int k = have ? div_by(en, q.by_tiles) : 0, t = have ? en - k * q.tiles : 0;
-    const int64_t slot = base + k * kstride + t;
+    slot[i] = have ? base + k * kstride + t : 0;  // entry 0 exists: the load needs no guard
+  }
 #pragma unroll
-    for (int f = 0; f < NF; ++f) e.v[i][f] = have ? ld_part<COH>(part + f * plane + slot) : (A)0;
+  for (int i = 0; i < kEarly; ++i) {
+#pragma unroll
+    for (int f = 0; f < NF; ++f) e.v[i][f] = ld_part<COH>(part + f * plane + slot[i]);
   }
 }
 // (count, mean, M2) entries -> merged triple (pivot form), available in every lane of the group's segment.
 template <typename A> __device__ __forceinline__ Moments<A> reduce_moments(const EarlyPartials<A, 3> &e) {
   A nl = (A)0, s1 = (A)0, s2 = (A)0;
-  const A kl = e.v[0][1];
+  const A kl = e.have(0) ? e.v[0][1] : (A)0;
 #pragma unroll
   for (int i = 0; i < kEarly; ++i) {
-    const A cn = e.v[i][0];
-    const A d = e.v[i][1] - kl;
+    const bool h = e.have(i);
+    const A cn = h ? e.v[i][0] : (A)0;
+    const A d = h ? e.v[i][1] - kl : (A)0;
     nl += cn;
     s1 += cn * d;
-    s2 += e.v[i][2] + cn * d * d;
+    s2 += (h ? e.v[i][2] : (A)0) + cn * d * d;
   }
   const A inv = nl > (A)0 ? (A)1 / nl : (A)0;
   const A mean_l = kl + s1 * inv;
@@ -207,7 +215,11 @@ template <typename A> __device__ __forceinline__ void reduce_sums(const EarlyPar
   ta = (A)0;
   tb = (A)0;
 #pragma unroll
-  for (int i = 0; i < kEarly; ++i) { ta += e.v[i][0]; tb += e.v[i][1]; }
+  for (int i = 0; i < kEarly; ++i) {
+    const bool h = e.have(i);
+    ta += h ? e.v[i][0] : (A)0;
+    tb += h ? e.v[i][1] : (A)0;
+  }
   segment_sum2(ta, tb, e.L);
 }
 // Channels [ca, cb) (relative to the chunk) of group g that lie inside the chunk.
@@ -642,14 +654,15 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
     const LanePos l = lane_pos(p, n, true);
     const int rows = l.rows;
     const int nb = block_batches<U>(p, l);
-    const int64_t off = (n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC;
+    const SafeLane sfl = safe_lane<VEC>(p, l, n);
+    const int64_t off = sfl.off;
     const int64_t step = (int64_t)p.rpi * p.C;
     typename LV::raw_t buf0[U], buf1[U];
     A sa[VEC], sb[VEC], unused1[VEC], unused2[VEC];
     auto issue = [&](auto sel, int bi) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const T *src = x + off + (int64_t)clamp_row(bi * U + u, rows) * step;
+        const T *src = x + off + (int64_t)clamp_row(bi * U + u, sfl.rows) * step;
         if constexpr (decltype(sel)::value == 0) buf0[u] = LV::load(src);
         else buf1[u] = LV::load(src);
       }
@@ -666,13 +679,15 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
       }
     };
     // order of issue: the few small loads the prologue depends on first, then the first batch of x, so that
-    // the small ones are not queued behind the bulk traffic of every workgroup
+    // the small ones are not queued behind the bulk traffic of every workgroup; no load of the prologue sits under
+    // a branch (idle lanes read valid addresses too), so each wait below covers exactly the loads it needs
+    // (the early fetch runs even when the general merge below will be used: a branch here would make the compiler
+    // wait for these loads before it issues the next ones)
     EarlyPartials<A, 3> early;
-    if (one_round) fetch_partials<A, 3, false>(early, part, group_plane(q, p.G, p.N), q, p, l);
-    if (rows > 0) {
-      lane_params<A, PT, VEC>(l, w, b, sa, sb);
-      issue(std::integral_constant<int, 0>{}, 0);
-    }
+    fetch_partials<A, 3, false>(early, part, group_plane(q, p.G, p.N), q, p, l);
+    lane_params_flat<A, PT, VEC>(sfl.c, w, b, part, sa, sb);
+    issue_order_fence();
+    issue(std::integral_constant<int, 0>{}, 0);
     if (one_round) {
       const Moments<A> m = reduce_moments<A>(early);
       if (early.valid && early.sl == 0) {
@@ -721,14 +736,15 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
     const LanePos l = lane_pos(p, n, false);
     const int rows = l.rows;
     const int nb = block_batches<U>(p, l);
-    const int64_t off = (n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC;
+    const SafeLane sfl = safe_lane<VEC>(p, l, n);
+    const int64_t off = sfl.off;
     const int64_t step = (int64_t)p.rpi * p.C;
     typename LV::raw_t bx0[U], bx1[U], bd0[U], bd1[U];
     A sa[VEC], sb[VEC], s1[VEC], s2[VEC], unused1[VEC], unused2[VEC];
     auto issue = [&](auto sel, int bi) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const int64_t o = off + (int64_t)clamp_row(bi * U + u, rows) * step;
+        const int64_t o = off + (int64_t)clamp_row(bi * U + u, sfl.rows) * step;
         if constexpr (decltype(sel)::value == 0) { bx0[u] = LV::load(x + o); bd0[u] = LV::load(dy + o); }
         else { bx1[u] = LV::load(x + o); bd1[u] = LV::load(dy + o); }
       }
@@ -748,14 +764,19 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
         }
       }
     };
-    // gamma of the channel this thread publishes in the epilogue, fetched now: off the tile's serial tail
-    const A gamma0 = (w && (int)threadIdx.x < l.wch) ? load_param<PT, A>(w, l.cstart + threadIdx.x) : (A)1;
-    // small loads first, then the bulk; the statistics are waited for on their own
+    // small loads first, then the bulk, none of them under a branch: the statistics are waited for on their own
     const StagedStats<A> st = fetch_chunk_stats<A>(mean, rstd, sdtype, p, l, sm_mu, sm_rs, partC);
-    if (rows > 0) {
-      lane_params<A, PT, VEC>(l, w, b, sa, sb);
-      issue(std::integral_constant<int, 0>{}, 0);
+    lane_params_flat<A, PT, VEC>(sfl.c, w, b, partC, sa, sb);
+    // gamma of the channel this thread publishes in the epilogue, fetched now: off the tile's serial tail
+    A gamma0;
+    {
+      const int cg = (int)threadIdx.x < l.wch ? threadIdx.x : 0;
+      const PT *gp = w ? (const PT *)w + l.cstart + cg : (const PT *)partC;
+      const A gv = load_param<PT, A>(gp, 0);
+      gamma0 = w ? gv : (A)1;
     }
+    issue_order_fence();
+    issue(std::integral_constant<int, 0>{}, 0);
     commit_chunk_stats<A>(st, l, sm_mu, sm_rs);
     __syncthreads();
 #pragma unroll
@@ -953,14 +974,15 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
     const LanePos l = lane_pos(p, n, true);
     const int rows = l.rows;
     const int nb = block_batches<U>(p, l);
-    const int64_t off = (n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC;
+    const SafeLane sfl = safe_lane<VEC>(p, l, n);
+    const int64_t off = sfl.off;
     const int64_t step = (int64_t)p.rpi * p.C;
     typename LV::raw_t bx0[U], bx1[U], bd0[U], bd1[U];
     A sa[VEC], sb[VEC], c1[VEC], c2[VEC];
     auto issue = [&](auto sel, int bi) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const int64_t o = off + (int64_t)clamp_row(bi * U + u, rows) * step;
+        const int64_t o = off + (int64_t)clamp_row(bi * U + u, sfl.rows) * step;
         if constexpr (decltype(sel)::value == 0) { bx0[u] = LV::load(x + o); bd0[u] = LV::load(dy + o); }
         else { bx1[u] = LV::load(x + o); bd1[u] = LV::load(dy + o); }
       }
@@ -981,17 +1003,17 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
     };
     EarlyPartials<A, 2> early;
     A emu = (A)0, ers = (A)0;
-    if (one_round) {
+    {
+      // unconditional, also when the general merge below will be used: a branch here would make the compiler wait
+      // for these loads before it issues the next ones
       fetch_partials<A, 2, false>(early, partG, plane, q, p, l);
-      if (early.valid && early.sl == 0) {
-        emu = load_scalar<A>(mean, n * p.G + l.g_lo + early.gi, sdtype);
-        ers = load_scalar<A>(rstd, n * p.G + l.g_lo + early.gi, sdtype);
-      }
+      const int64_t gidx = early.valid ? n * p.G + l.g_lo + early.gi : 0;  // entry 0 exists: no guard on the loads
+      emu = load_scalar_flat<A>(mean, gidx, sdtype, partC);
+      ers = load_scalar_flat<A>(rstd, gidx, sdtype, partC);
     }
-    if (rows > 0) {
-      lane_params<A, PT, VEC>(l, w, b, sa, sb);
-      issue(std::integral_constant<int, 0>{}, 0);  // in flight while the group sums are merged
-    }
+    lane_params_flat<A, PT, VEC>(sfl.c, w, b, partC, sa, sb);
+    issue_order_fence();
+    issue(std::integral_constant<int, 0>{}, 0);  // in flight while the group sums are merged
     if (one_round) {
       A ta, tb;
       reduce_sums<A>(early, ta, tb);
