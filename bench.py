@@ -204,7 +204,8 @@ def kernel_profile(probs, steps):
             for _ in range(steps):
                 p.step(0, stream)
             res = _cabi.profile_collect()
-            out[p.cfg.name] = {k: ms / n * 1e3 for k, (n, ms) in res.items() if n}
+            # mean per launch, and launches per call (a call may run one kernel kind several times, over groups of samples)
+            out[p.cfg.name] = {k: (ms / n * 1e3, n / steps) for k, (n, ms) in res.items() if n}
     finally:
         _cabi.profile_enable(False)
     return out
@@ -366,9 +367,13 @@ def main():
     # ---- per-kernel durations (HIP events on the launch stream) ----
     prof = kernel_profile(probs, max(20, args.steps // 4))
     S_of = {p.cfg.name: p.S for p in probs}
-    dom_shape, dominant = max(((n, k) for n in prof for k in prof[n]), key=lambda nk: prof[nk[0]][nk[1]])
-    dom_us = prof[dom_shape][dominant]
-    dom_bytes = KERNEL_STREAMS[dominant] * S_of[dom_shape]
+
+    def launch_bytes(name, kind):  # algorithmic bytes of ONE launch of this kind on this shape
+        return KERNEL_STREAMS[kind] * S_of[name] / prof[name][kind][1]
+
+    dom_shape, dominant = max(((n, k) for n in prof for k in prof[n]), key=lambda nk: prof[nk[0]][nk[1]][0])
+    dom_us = prof[dom_shape][dominant][0]
+    dom_bytes = launch_bytes(dom_shape, dominant)
     achieved = dom_bytes / (dom_us * 1e-6) / 1e9
     traffic = recorded_traffic()
     tr = traffic.get((dom_shape, dominant))
@@ -384,10 +389,10 @@ def main():
         "traffic_source": "profiles/hbm_traffic_sd_unet.txt (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, copy-calibrated)" if tr else None,
         "bytes_per_launch": dom_bytes,
         "mean_launch_us": round(dom_us, 3),
-        "kernels": {n: {k: {"us": round(us, 3), "alg_bytes": KERNEL_STREAMS[k] * S_of[n],
-                            "frac": round(KERNEL_STREAMS[k] * S_of[n] / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+        "kernels": {n: {k: {"us": round(us, 3), "launches_per_call": per_call, "alg_bytes": launch_bytes(n, k),
+                            "frac": round(launch_bytes(n, k) / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
                             "traffic": (round(sum(traffic[(n, k)])) if (n, k) in traffic else None)}
-                        for k, us in kinds.items()} for n, kinds in prof.items()},
+                        for k, (us, per_call) in kinds.items()} for n, kinds in prof.items()},
     }
 
     # ---- per-shape table ----

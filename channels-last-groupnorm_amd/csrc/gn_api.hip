@@ -167,7 +167,7 @@ size_t fwd_ws_bytes(int64_t N, int64_t R, int64_t C, int64_t G, int dtype) {
     if (v > need) need = v;
     resident = dtype == GN_F64 ? 0 : resident_fwd_bytes(G);
   }
-  return max_size(need * acc_size(dtype), resident);
+  return max_size(kWorkspaceHeader + need * acc_size(dtype), resident);
 }
 size_t bwd_ws_bytes(int64_t N, int64_t R, int64_t C, int64_t G, int dtype) {
   const int vec = 16 / elem_size(dtype);
@@ -179,7 +179,7 @@ size_t bwd_ws_bytes(int64_t N, int64_t R, int64_t C, int64_t G, int dtype) {
     if (v > need) need = v;
     resident = dtype == GN_F64 ? 0 : resident_bwd_bytes((int64_t)pv.lpr * vec, G);
   }
-  return max_size(need * acc_size(dtype), resident);
+  return max_size(kWorkspaceHeader + need * acc_size(dtype), resident);
 }
 
 __global__ void fill_zero_kernel(void *p, int64_t n, int dtype) {

@@ -38,7 +38,7 @@ struct SyncArea {
   unsigned rec_bytes;
   unsigned long long *flags;  // [N][nchunk][tiles]
   unsigned long long epoch;   // value that marks "written in this call"
-  const unsigned long long *generation;  // optional device word folded into the epoch (see resident_epoch)
+  const unsigned long long *generation;  // device counter that replaces the epoch in captured launches (resident_epoch)
   unsigned long long *status; // set to the epoch if a wait of this call timed out
   int max_spins;              // polls allowed per wait
   unsigned long long *trace;  // optional [workgroup][kTracePoints] timestamps (100 MHz wall clock), else null
@@ -59,10 +59,14 @@ __device__ __forceinline__ void trace_point(const SyncArea &s, int point, float 
 
 // A launch recorded into a HIP graph is replayed with identical kernel arguments, so the host cannot give
 // each replay a fresh epoch.  For captured launches the host therefore records a one-thread kernel in front
-// that increments a generation word in the workspace, and the epoch becomes host value + generation * odd.
+// that increments a generation word in the workspace header, and that counter is the epoch: it is different
+// for every captured launch that ever runs on this workspace, whatever graph it belongs to.  Bit 63 keeps the
+// two families apart: set for counter epochs, clear for the host's.
 template <int UNUSED> __global__ void bump_generation_kernel(unsigned long long *generation) { *generation += 1; }
 __device__ __forceinline__ SyncArea resident_epoch(SyncArea s) {
-  if (s.generation) s.epoch += *s.generation * 0x9E3779B97F4A7C15ull;
+  constexpr unsigned long long kCaptured = 1ull << 63;
+  if (s.generation) s.epoch = kCaptured | *s.generation;
+  else s.epoch &= ~kCaptured;
   if (s.epoch == 0) s.epoch = 1;
   return s;
 }
@@ -313,7 +317,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 8 
 template <typename T, typename PT, int VEC, int ACT, int NV>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 ? 4 : NV <= 8 ? 3 : NV <= 16 ? 2 : 1))) void fused_bwd_kernel(
     const T *__restrict__ x, const T *__restrict__ dy, T *__restrict__ dx, const void *mean, const void *rstd, int sdtype,
-    const void *w, const void *b, acc_t<T> *__restrict__ partC, SyncArea sync_arg, void *dw, void *db, Plan p) {
+    const void *w, const void *b, acc_t<T> *__restrict__ partC, SyncArea sync_arg, void *dw, void *db,
+    const acc_t<T> *partC_all, const void *mean_all, const void *rstd_all, int64_t n_all, Plan p) {
   using A = acc_t<T>;
   using LV = LaneVec<T, VEC>;
   const SyncArea sync = resident_epoch(sync_arg);
@@ -469,11 +474,14 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
     }
   }
   trace_point(sync, 4);
-  // dgamma / dbeta (compute_dweight_dbias, gn_kernel.cu:695-728): the workgroups of sample 0 share the
-  // channels of their chunk, a segment of L lanes per channel summing over every (sample, row tile) pair,
-  // once all those tiles have published their per-channel sums.  The dx stores above drain meanwhile.
+  // dgamma / dbeta (compute_dweight_dbias, gn_kernel.cu:695-728): the workgroups of this launch's first sample
+  // share the channels of their chunk, a segment of L lanes per channel summing over every (sample, row tile)
+  // pair, once all tiles of this launch have published their per-channel sums.  The dx stores above drain
+  // meanwhile.  When the tensor is run as several launches over groups of samples only the last one gets dw / db;
+  // it sums over all n_all samples (partC_all, mean_all, rstd_all are the whole tensor's; the earlier launches
+  // have completed, so their sums need no flag).
   if (n == 0 && (dw || db)) {
-    const int pairs = (int)p.N * p.tiles;
+    const int pairs = (int)n_all * p.tiles;
     const int L = pow2_ceil_clamped(pairs, 64);
     const int cpp = kBlock >> __builtin_ctz(L);  // channels per pass of the workgroup (L is a power of two)
     const int slot = threadIdx.x >> __builtin_ctz(L), sl = threadIdx.x & (L - 1);
@@ -487,13 +495,13 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
         if (valid) {
           const int g = div_by(c, p.by_D);
           for (int e = sl; e < pairs; e += L) {
-            const int64_t nn = div_by(e, p.by_tiles);
+            const int64_t nn = e / p.tiles;
             const int t = e - (int)nn * p.tiles;
             const int64_t idx = ((nn * p.tiles + t) * p.C + c) * 2;
-            const A s1 = ld_part<true>(partC + idx);
-            const A s2 = ld_part<true>(partC + idx + 1);
-            const A mu = load_scalar<A>(mean, nn * p.G + g, sdtype);
-            const A rs = load_scalar<A>(rstd, nn * p.G + g, sdtype);
+            const A s1 = ld_part<true>(partC_all + idx);
+            const A s2 = ld_part<true>(partC_all + idx + 1);
+            const A mu = load_scalar<A>(mean_all, nn * p.G + g, sdtype);
+            const A rs = load_scalar<A>(rstd_all, nn * p.G + g, sdtype);
             t1 += (s1 - mu * s2) * rs;
             t2 += s2;
           }

@@ -64,14 +64,28 @@ inline BwdWorkspace bwd_workspace(const Plan &p) {
   w.total = w.compactG + align_up((size_t)p.N * p.G * 2, 64);
   return w;
 }
+// Every layout of the workspace (streaming or single-launch, forward or backward) leaves its first 256 bytes
+// alone: they hold the generation word of captured single-launch kernels, which must survive whatever else a
+// caller runs on the same workspace between two replays of a graph.
+constexpr size_t kWorkspaceHeader = 256;
 // The resident kernels keep their partial results and one flag per workgroup in the same workspace.
 constexpr int kMaxResidentBlocks = 4 * kNumCU;
 inline size_t resident_rec_bytes(int64_t G) { return (size_t)16 * G * kMaxResidentBlocks; }
-inline size_t resident_fwd_bytes(int64_t G) { return align_up(resident_rec_bytes(G), 256) + 256; }
+inline size_t resident_fwd_bytes(int64_t G) { return kWorkspaceHeader + align_up(resident_rec_bytes(G), 256); }
 // chunk_channels = channels per workgroup (lpr * vec): N * tiles * C = workgroups * chunk_channels
+// A tensor of several samples that is too large for one single-launch kernel may still be run as up to
+// kMaxBatches such launches over consecutive groups of samples (samples share nothing but dgamma / dbeta).
+constexpr int kMaxBatches = 4;
+// Per-channel tile sums of the backward, [N][tiles][C][2] floats: one launch's worth at most
+// 2 * chunk_channels * kMaxResidentBlocks, and room for the launches of a batched call up to a fixed bound.
+inline size_t resident_partc_bytes(int64_t chunk_channels) {
+  const size_t one = (size_t)2 * chunk_channels * kMaxResidentBlocks * 4;
+  const size_t many = one * kMaxBatches < ((size_t)8 << 20) ? one * kMaxBatches : ((size_t)8 << 20);
+  return align_up(one > many ? one : many, 256);
+}
 inline size_t resident_bwd_bytes(int64_t chunk_channels, int64_t G) {
-  return align_up((size_t)2 * chunk_channels * kMaxResidentBlocks * 4, 256) + align_up(resident_rec_bytes(G), 256) +
-         (size_t)kMaxResidentBlocks * 8 + 256;
+  return kWorkspaceHeader + resident_partc_bytes(chunk_channels) + align_up(resident_rec_bytes(G), 256) +
+         (size_t)kMaxResidentBlocks * 8;
 }
 // A fresh nonzero 64-bit value per call (gn_api.hip).
 unsigned long long next_epoch();

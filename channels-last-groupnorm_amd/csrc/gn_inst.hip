@@ -75,13 +75,14 @@ template <typename K> int resident_slots(K kernel) {
 // Row tiling of a resident launch with a register capacity of nv rows per lane: tiles of exactly nv rows per
 // lane (all loads useful; only the last tile of a sample may be short), every workgroup resident.
 // Returns false if it does not fit.
-bool resident_tiling(const Plan &base, int nv, int slots, Plan &out) {
-  const int64_t columns = base.N * base.nchunk;
-  if (slots <= 0 || columns > slots || base.N > 65535) return false;
+bool resident_tiling(const Plan &base, int64_t samples, int nv, int slots, Plan &out) {
+  const int64_t columns = samples * base.nchunk;
+  if (slots <= 0 || columns > slots || samples > 65535) return false;
   const int64_t rows = (int64_t)nv * base.rpi;
   const int64_t tiles = (base.R + rows - 1) / rows;
   if (columns * tiles > slots) return false;
   out = base;
+  out.N = samples;
   out.tile_rows = (int)rows;
   out.tiles = (int)tiles;
   out.nblocks = columns * tiles;
@@ -92,7 +93,7 @@ bool resident_tiling(const Plan &base, int nv, int slots, Plan &out) {
 struct ResidentWorkspace {
   A *partC;  // backward only
   SyncArea sync;
-  unsigned long long *generation;  // device word behind the records / flags
+  unsigned long long *generation;  // device word in the workspace header
 };
 // True while `stream` is recording into a HIP graph.
 bool stream_is_capturing(hipStream_t stream) {
@@ -113,13 +114,13 @@ void arm_generation(ResidentWorkspace &r, hipStream_t stream) {
 }
 ResidentWorkspace resident_fwd_ws(void *ws, const Plan &p) {
   ResidentWorkspace r;
-  char *base = (char *)ws;
+  char *base = (char *)ws + kWorkspaceHeader;
   r.partC = nullptr;
   r.sync.recs = base;
   r.sync.rec_bytes = (unsigned)resident_rec_bytes(p.G);
   r.sync.flags = nullptr;
   r.sync.status = resident_status();
-  r.generation = (unsigned long long *)(base + align_up(resident_rec_bytes(p.G), 256));
+  r.generation = (unsigned long long *)ws;
   r.sync.max_spins = resident_spin_limit();
   r.sync.epoch = next_epoch();
   r.sync.trace = trace_buffer();
@@ -128,16 +129,16 @@ ResidentWorkspace resident_fwd_ws(void *ws, const Plan &p) {
 }
 ResidentWorkspace resident_bwd_ws(void *ws, const Plan &p) {
   ResidentWorkspace r;
-  char *base = (char *)ws;
+  char *base = (char *)ws + kWorkspaceHeader;
   const size_t cc = (size_t)p.lpr * p.vec;
   r.partC = (A *)base;
-  char *recs = base + align_up((size_t)2 * cc * kMaxResidentBlocks * 4, 256);
+  char *recs = base + resident_partc_bytes(cc);
   r.sync.recs = recs;
   r.sync.rec_bytes = (unsigned)resident_rec_bytes(p.G);
   char *f = recs + align_up(resident_rec_bytes(p.G), 256);
   r.sync.flags = (unsigned long long *)f;
   r.sync.status = resident_status();
-  r.generation = (unsigned long long *)(f + (size_t)kMaxResidentBlocks * 8);
+  r.generation = (unsigned long long *)ws;
   r.sync.max_spins = resident_spin_limit();
   r.sync.epoch = next_epoch();
   r.sync.trace = trace_buffer();
@@ -145,23 +146,49 @@ ResidentWorkspace resident_bwd_ws(void *ws, const Plan &p) {
   return r;
 }
 
-template <typename PT, int ACT, int NV> bool try_resident_fwd_nv(const FwdArgs &a) {
+// How many consecutive single-launch kernels over groups of samples still beat the streaming pair.  Each launch
+// pays a fixed latency of roughly 9 microseconds in the backward but moves 3 S bytes instead of the pair's 5 S
+// (about 5.4 bytes per nanosecond either way, and about 14 us fixed for the pair); measured on (N, 320, 128, 128)
+// bf16: two launches equal the pair at N = 4 and beat it by 14 % at N = 6, three launches by 6 % at N = 8.
+// In the forward the pair only moves 3 S against 2 S, and two launches measured 5 % slower than the pair: never split.
+int worthwhile_batches(const Plan &p, bool backward) {
+  if (!backward) return 1;
+  const double s_mb = (double)p.N * p.R * p.C * sizeof(elem_t) / 1e6;
+  const double k = (14.0 + 0.405 * s_mb) / 9.0;
+  const int kk = k < 1.0 ? 1 : (int)k;
+  return kk < kMaxBatches ? kk : kMaxBatches;
+}
+size_t stat_size(int sdtype) { return sdtype == GN_F32 ? 4 : sdtype == GN_F64 ? 8 : 2; }
+
+// One NV variant, the tensor cut into `batches` launches over consecutive samples (1: the whole tensor).
+template <typename PT, int ACT, int NV> bool try_resident_fwd_nv(const FwdArgs &a, int batches) {
   if (NV < resident_min_rows()) return false;
   auto kernel = fused_fwd_kernel<elem_t, PT, kVec, ACT, NV>;
   static const int slots = resident_slots(kernel);
+  const int64_t per = (a.plan.N + batches - 1) / batches;
   Plan p;
-  if (!resident_tiling(a.plan, NV, slots, p)) return false;
-  ResidentWorkspace r = resident_fwd_ws(a.ws, p);
-  if (!r.sync.status) return false;
+  if (!resident_tiling(a.plan, per, NV, slots, p)) return false;
+  if (!resident_status()) return false;
   mark_resident_launch();
-  arm_generation(r, a.stream);
-  launch(kKindFusedFwd, kernel, tile_grid(p, 0), dim3(kBlock), a.stream, (const elem_t *)a.x, (elem_t *)a.y, r.sync, a.w, a.b,
-                     a.mean, a.rstd, a.sdtype, (A)a.eps, p);
+  const int64_t sample = a.plan.R * a.plan.C;
+  for (int64_t n0 = 0; n0 < a.plan.N; n0 += per) {
+    Plan pb = p;
+    if (a.plan.N - n0 < per) resident_tiling(a.plan, a.plan.N - n0, NV, slots, pb);  // the last, shorter group
+    ResidentWorkspace r = resident_fwd_ws(a.ws, pb);  // the launches follow each other on the stream: same records
+    arm_generation(r, a.stream);
+    launch(kKindFusedFwd, kernel, tile_grid(pb, 0), dim3(kBlock), a.stream, (const elem_t *)a.x + n0 * sample,
+           (elem_t *)a.y + n0 * sample, r.sync, a.w, a.b, (char *)a.mean + n0 * a.plan.G * stat_size(a.sdtype),
+           (char *)a.rstd + n0 * a.plan.G * stat_size(a.sdtype), a.sdtype, (A)a.eps, pb);
+  }
   return true;
 }
 template <typename PT, int ACT> bool try_resident_fwd_act(const FwdArgs &a) {
-  return try_resident_fwd_nv<PT, ACT, 4>(a) || try_resident_fwd_nv<PT, ACT, 8>(a) || try_resident_fwd_nv<PT, ACT, 16>(a) ||
-         try_resident_fwd_nv<PT, ACT, 32>(a);
+  const int most = a.plan.N < worthwhile_batches(a.plan, false) ? (int)a.plan.N : worthwhile_batches(a.plan, false);
+  for (int b = 1; b <= most; ++b)
+    if (try_resident_fwd_nv<PT, ACT, 4>(a, b) || try_resident_fwd_nv<PT, ACT, 8>(a, b) ||
+        try_resident_fwd_nv<PT, ACT, 16>(a, b) || try_resident_fwd_nv<PT, ACT, 32>(a, b))
+      return true;
+  return false;
 }
 template <typename PT> bool try_resident_fwd_pt(const FwdArgs &a) {
   switch (a.act) {
@@ -177,23 +204,42 @@ bool try_resident_fwd(const FwdArgs &a) {
   return a.pdtype == GN_INST_DTYPE ? try_resident_fwd_pt<elem_t>(a) : try_resident_fwd_pt<wide_param_t>(a);
 }
 
-template <typename PT, int ACT, int NV> bool try_resident_bwd_nv(const BwdArgs &a) {
+template <typename PT, int ACT, int NV> bool try_resident_bwd_nv(const BwdArgs &a, int batches) {
   if (NV < resident_min_rows()) return false;
   auto kernel = fused_bwd_kernel<elem_t, PT, kVec, ACT, NV>;
   static const int slots = resident_slots(kernel);
+  const int64_t per = (a.plan.N + batches - 1) / batches;
   Plan p;
-  if (!resident_tiling(a.plan, NV, slots, p)) return false;
-  ResidentWorkspace r = resident_bwd_ws(a.ws, p);
-  if (!r.sync.status) return false;
+  if (!resident_tiling(a.plan, per, NV, slots, p)) return false;
+  // per-channel tile sums of every sample stay in the workspace until the last launch has summed them
+  const size_t partc_need = (size_t)a.plan.N * p.tiles * a.plan.C * 2 * sizeof(A);
+  if (partc_need > resident_partc_bytes((int64_t)p.lpr * p.vec)) return false;
+  if (!resident_status()) return false;
   mark_resident_launch();
-  arm_generation(r, a.stream);
-  launch(kKindFusedBwd, kernel, tile_grid(p, 0), dim3(kBlock), a.stream, (const elem_t *)a.x, (const elem_t *)a.dy,
-                     (elem_t *)a.dx, a.mean, a.rstd, a.sdtype, a.w, a.b, r.partC, r.sync, a.dw, a.db, p);
+  const int64_t sample = a.plan.R * a.plan.C;
+  const size_t ssz = stat_size(a.sdtype);
+  for (int64_t n0 = 0; n0 < a.plan.N; n0 += per) {
+    Plan pb = p;
+    if (a.plan.N - n0 < per) resident_tiling(a.plan, a.plan.N - n0, NV, slots, pb);  // the last, shorter group
+    pb.tiles = p.tiles;  // same row tiling in every group (it depends on R and NV only)
+    ResidentWorkspace r = resident_bwd_ws(a.ws, pb);
+    arm_generation(r, a.stream);
+    const bool last = n0 + per >= a.plan.N;
+    A *partC_here = r.partC + n0 * p.tiles * a.plan.C * 2;
+    launch(kKindFusedBwd, kernel, tile_grid(pb, 0), dim3(kBlock), a.stream, (const elem_t *)a.x + n0 * sample,
+           (const elem_t *)a.dy + n0 * sample, (elem_t *)a.dx + n0 * sample, (const char *)a.mean + n0 * a.plan.G * ssz,
+           (const char *)a.rstd + n0 * a.plan.G * ssz, a.sdtype, a.w, a.b, partC_here, r.sync, last ? a.dw : nullptr,
+           last ? a.db : nullptr, (const A *)r.partC, a.mean, a.rstd, a.plan.N, pb);
+  }
   return true;
 }
 template <typename PT, int ACT> bool try_resident_bwd_act(const BwdArgs &a) {
-  return try_resident_bwd_nv<PT, ACT, 4>(a) || try_resident_bwd_nv<PT, ACT, 8>(a) || try_resident_bwd_nv<PT, ACT, 16>(a) ||
-         try_resident_bwd_nv<PT, ACT, 32>(a);
+  const int most = a.plan.N < worthwhile_batches(a.plan, true) ? (int)a.plan.N : worthwhile_batches(a.plan, true);
+  for (int b = 1; b <= most; ++b)
+    if (try_resident_bwd_nv<PT, ACT, 4>(a, b) || try_resident_bwd_nv<PT, ACT, 8>(a, b) ||
+        try_resident_bwd_nv<PT, ACT, 16>(a, b) || try_resident_bwd_nv<PT, ACT, 32>(a, b))
+      return true;
+  return false;
 }
 template <typename PT> bool try_resident_bwd_pt(const BwdArgs &a) {
   switch (a.act) {
@@ -213,7 +259,7 @@ template <int VEC> hipError_t fwd_impl(const FwdArgs &a) {
   if (VEC != 1 && try_resident_fwd(a)) return hipGetLastError();
   const Plan &p = a.plan;
   const FwdWorkspace ws = fwd_workspace(p);
-  A *base = (A *)a.ws;
+  A *base = (A *)((char *)a.ws + kWorkspaceHeader);
   A *part = base + ws.part, *compact = base + ws.compact;
   PartialGeo q = producer_geo(p);
   {
@@ -237,7 +283,7 @@ template <int VEC> hipError_t fwd_impl(const FwdArgs &a) {
 template <typename PT, int VEC, int ACT> void launch_bwd_act(const BwdArgs &a) {
   const Plan &p = a.plan;
   const BwdWorkspace ws = bwd_workspace(p);
-  A *base = (A *)a.ws;
+  A *base = (A *)((char *)a.ws + kWorkspaceHeader);
   A *partC = base + ws.partC, *partG = base + ws.partG, *compactC = base + ws.compactC, *compactG = base + ws.compactG;
   PartialGeo q = producer_geo(p);
   {

@@ -419,3 +419,49 @@ def test_single_launch_timeout_is_reported(device):
         assert err(mean2, truth["mean"]) <= 1e-5 and err(y2, truth["y"]) <= 2.0 ** -7
     finally:
         _cabi.set_resident(before)
+
+
+@pytest.mark.parametrize("shape,G", [((2, 64, 23, 19), 8), ((1, 1280, 64, 64), 32), ((5, 320, 128, 128), 32)])
+def test_hip_graph_replay(family, shape, G, device):
+    """Forward + backward recorded into a HIP graph through the C ABI and replayed several times, with eager calls
+    on the same workspaces and synchronisations in between; every replay must reproduce the eager result bit for bit
+    (the largest shape runs as several single-launch kernels over groups of samples)."""
+    gen = torch.Generator().manual_seed(21)
+    N, C = shape[0], shape[1]
+    x = nrc_view(channels_last_like(shape, torch.bfloat16, device, gen, 1.5, 0.3))
+    dy = nrc_view(channels_last_like(shape, torch.bfloat16, device, gen))
+    w = (torch.rand(C, generator=gen) + 0.5).to(torch.bfloat16).to(device)
+    b = (0.1 * torch.randn(C, generator=gen)).to(torch.bfloat16).to(device)
+    lib = _cabi.lib
+    R = x.shape[1]
+    ws_f = torch.empty((lib.gnnhwc_fwd_workspace_bytes(N, R, C, G, 3),), dtype=torch.uint8, device=device)
+    ws_b = torch.empty((lib.gnnhwc_bwd_workspace_bytes(N, R, C, G, 3),), dtype=torch.uint8, device=device)
+    y = torch.empty_like(x)
+    dx = torch.empty_like(x)
+
+    def step():
+        _, mean, rstd = cabi_fwd(x, w, b, G, 1e-5, 2, y=y, ws=ws_f)
+        _, dw, db = cabi_bwd(dy, x, w, b, mean, rstd, G, 2, dx=dx, ws=ws_b)
+        return mean, rstd, dw, db
+
+    mean, rstd, dw, db = step()
+    torch.cuda.synchronize()
+    want = [t.clone() for t in (y, dx, mean, rstd, dw, db)]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        mean_g, rstd_g, dw_g, db_g = step()
+    for rep in range(4):
+        for t in (y, dx, mean_g, rstd_g, dw_g, db_g):
+            t.fill_(float("nan"))
+        g.replay()
+        torch.cuda.synchronize()
+        for name, got, ref in zip(("y", "dx", "mean", "rstd", "dw", "db"), (y, dx, mean_g, rstd_g, dw_g, db_g), want):
+            assert torch.equal(got, ref), "replay %d: %s differs from the eager result" % (rep, name)
+        step()  # eager work on the same workspaces between replays
+        torch.cuda.synchronize()
