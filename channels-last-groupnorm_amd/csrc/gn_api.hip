@@ -352,7 +352,7 @@ int gnnhwc_fwd(const void *x, const void *weight, const void *bias, void *y, voi
   if (N == 0 || R == 0) return GNNHWC_OK;  // nothing to normalise; mean / rstd of an empty slab are left untouched
   rc = check_resident_health();
   if (rc != GNNHWC_OK) return rc;
-  if (!x || !y || !mean || !rstd) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "x, y, mean and rstd must not be null");
+  if (!x || !y) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "x and y must not be null");
   const size_t need = gnnhwc_fwd_workspace_bytes(N, R, C, G, dtype);
   if (!workspace || !aligned16(workspace) || workspace_bytes < need)
     return fail(GNNHWC_ERR_WORKSPACE, "forward workspace must be 16-byte aligned and at least %zu bytes (got %p, %zu bytes)",

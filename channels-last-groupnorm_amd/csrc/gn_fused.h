@@ -283,8 +283,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 8 
         sm0[gi] = gmean;
         sm1[gi] = rs;
         if (l.tile == 0 && g * p.D >= l.cstart) {
-          store_scalar<A>(mean_out, n * p.G + g, sdtype, gmean);
-          store_scalar<A>(rstd_out, n * p.G + g, sdtype, rs);
+          if (mean_out) store_scalar<A>(mean_out, n * p.G + g, sdtype, gmean);
+          if (rstd_out) store_scalar<A>(rstd_out, n * p.G + g, sdtype, rs);
         }
       }
     }

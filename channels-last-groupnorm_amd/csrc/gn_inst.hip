@@ -177,8 +177,8 @@ template <typename PT, int ACT, int NV> bool try_resident_fwd_nv(const FwdArgs &
     ResidentWorkspace r = resident_fwd_ws(a.ws, pb);  // the launches follow each other on the stream: same records
     arm_generation(r, a.stream);
     launch(kKindFusedFwd, kernel, tile_grid(pb, 0), dim3(kBlock), a.stream, (const elem_t *)a.x + n0 * sample,
-           (elem_t *)a.y + n0 * sample, r.sync, a.w, a.b, (char *)a.mean + n0 * a.plan.G * stat_size(a.sdtype),
-           (char *)a.rstd + n0 * a.plan.G * stat_size(a.sdtype), a.sdtype, (A)a.eps, pb);
+           (elem_t *)a.y + n0 * sample, r.sync, a.w, a.b, a.mean ? (char *)a.mean + n0 * a.plan.G * stat_size(a.sdtype) : nullptr,
+           a.rstd ? (char *)a.rstd + n0 * a.plan.G * stat_size(a.sdtype) : nullptr, a.sdtype, (A)a.eps, pb);
   }
   return true;
 }

@@ -521,8 +521,8 @@ __device__ __forceinline__ void merge_chunk_stats(const A *__restrict__ part, co
       sm_mu[gi] = m.mean;
       sm_rs[gi] = rs;
       if (l.tile == 0 && g * p.D >= l.cstart) {  // the chunk where the group starts reports it
-        store_scalar<A>(mean_out, l.n * p.G + g, sdtype, m.mean);
-        store_scalar<A>(rstd_out, l.n * p.G + g, sdtype, rs);
+        if (mean_out) store_scalar<A>(mean_out, l.n * p.G + g, sdtype, m.mean);
+        if (rstd_out) store_scalar<A>(rstd_out, l.n * p.G + g, sdtype, rs);
       }
     }
   }
@@ -696,8 +696,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
         sm_mu[early.gi] = m.mean;
         sm_rs[early.gi] = rs;
         if (l.tile == 0 && g * p.D >= l.cstart) {  // the chunk where the group starts reports it
-          store_scalar<A>(mean_out, n * p.G + g, sdtype, m.mean);
-          store_scalar<A>(rstd_out, n * p.G + g, sdtype, rs);
+          if (mean_out) store_scalar<A>(mean_out, n * p.G + g, sdtype, m.mean);
+          if (rstd_out) store_scalar<A>(rstd_out, n * p.G + g, sdtype, rs);
         }
       }
       __syncthreads();

@@ -83,6 +83,8 @@ size_t gnnhwc_bwd_workspace_bytes(int64_t N, int64_t R, int64_t C, int64_t G, in
  *                  custom_gn.cpp:35; here GNNHWC_F32 parameters with F16/BF16 data are also accepted).
  *   stats_dtype  : type mean / rstd are written in; equal to dtype, or GNNHWC_F32 for F16/BF16 data.
  * Statistics are always accumulated and applied in fp32 (fp64 for F64) whatever stats_dtype is.
+ * Inference: mean and / or rstd may be NULL when the caller does not need them (no backward will follow), and
+ * y may be the same buffer as x (every element of x is read before the element of y that replaces it is written).
  */
 int gnnhwc_fwd(const void *x, const void *weight, const void *bias,
                void *y, void *mean, void *rstd,

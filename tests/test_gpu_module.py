@@ -387,6 +387,30 @@ def test_reference_brute_force_sample(family, B, C, R, G, device):
     check_against_torch(x, G, "identity", w, b, dy)
 
 
+@pytest.mark.parametrize("shape,G", [((2, 64, 23, 19), 8), ((4, 320, 128, 128), 32)])
+def test_inference_in_place_without_statistics(family, shape, G, device):
+    """Forward with y aliasing x and no mean / rstd outputs gives the same y as the ordinary call."""
+    import ctypes
+
+    gen = torch.Generator().manual_seed(31)
+    C = shape[1]
+    x = nrc_view(channels_last_like(shape, torch.bfloat16, device, gen, 1.5, 0.3))
+    w = (torch.rand(C, generator=gen) + 0.5).to(torch.bfloat16).to(device)
+    b = (0.1 * torch.randn(C, generator=gen)).to(torch.bfloat16).to(device)
+    y_ref, _, _ = cabi_fwd(x, w, b, G, 1e-5, 2)
+    N, R, _ = x.shape
+    lib = _cabi.lib
+    nbytes = lib.gnnhwc_fwd_workspace_bytes(N, R, C, G, 3)
+    ws = torch.empty((nbytes,), dtype=torch.uint8, device=device)
+    buf = x.clone()
+    vp = lambda t: ctypes.c_void_p(t.data_ptr())  # noqa: E731
+    rc = lib.gnnhwc_fwd(vp(buf), vp(w), vp(b), vp(buf), None, None, N, R, C, G, 1e-5, 2, 3, 3, 0, vp(ws), nbytes,
+                        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    _cabi.check(rc, "gnnhwc_fwd")
+    torch.cuda.synchronize()
+    assert torch.equal(buf, y_ref)
+
+
 def test_single_launch_timeout_is_reported(device):
     """A single-launch kernel whose workgroups cannot wait for each other (forced here from the host with a poll
     limit of 0, so every kernel still ends normally) leaves invalid output; the next call must say so, and the
