@@ -434,6 +434,9 @@ def main():
                    "timing": "HIP graph replay of the K steps" if use_graph else "eager launches through the C ABI",
                    "algorithmic_bytes_per_step": alg},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
+        # the reference's own benchmark counts 3 tensor sizes for a forward and 8 for forward + backward
+        # (benchmark.py:101,107); the same time expressed in that accounting, for comparison with its CSVs
+        "reference_accounting_gbps": round(sum((8 if p.bwd else 3) * p.S for p in probs) / (t / args.steps) / 1e9, 1),
         ("eager_ms_per_step" if use_graph else "graph_replay_ms_per_step"): round(t_other / args.steps * 1e3, 5),
         "roofline": roofline,
         "shapes": shapes,
