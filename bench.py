@@ -201,11 +201,16 @@ def kernel_profile(probs, steps):
             for _ in range(steps):  # untimed pass: creates the event pool, so that the host keeps ahead of the GPU below
                 p.step(0, stream)
             _cabi.profile_collect()
-            for _ in range(steps):
-                p.step(0, stream)
-            res = _cabi.profile_collect()
+            best = {}
+            for _ in range(3):  # three passes, the fastest mean of each kind: robust against a transient slow start
+                for _ in range(steps):
+                    p.step(0, stream)
+                res = _cabi.profile_collect()
+                for k, (n, ms) in res.items():
+                    if n and (k not in best or ms / n < best[k][0] / best[k][1]):
+                        best[k] = (ms, n)
             # mean per launch, and launches per call (a call may run one kernel kind several times, over groups of samples)
-            out[p.cfg.name] = {k: (ms / n * 1e3, n / steps) for k, (n, ms) in res.items() if n}
+            out[p.cfg.name] = {k: (ms / n * 1e3, n / steps) for k, (ms, n) in best.items()}
     finally:
         _cabi.profile_enable(False)
     return out
