@@ -31,12 +31,14 @@ namespace gn {
 
 constexpr int kMaxSpins = 1 << 22;  // default bound on the polls of one wait (seconds of polling)
 constexpr int kRecFast = 4;
+constexpr int kTailFast = 2;  // channel records a lane of the dgamma / dbeta stage requests ahead of the dx phase
 constexpr int kMaxResidentBlocksDev = 4 * kNumCU;  // records a lane keeps in registers while polling
 
 struct SyncArea {
   void *recs;                 // 16-byte records, laid out [N][nchunk][G][tiles]
   unsigned rec_bytes;
-  unsigned long long *flags;  // [N][nchunk][tiles]
+  void *crecs;                // backward: 16-byte records {S1, S2, epoch} per (sample, tile, channel) of the whole tensor
+  unsigned crec_bytes;
   unsigned long long epoch;   // value that marks "written in this call"
   const unsigned long long *generation;  // device counter that replaces the epoch in captured launches (resident_epoch)
   unsigned long long *status; // set to the epoch if a wait of this call timed out
@@ -71,14 +73,13 @@ __device__ __forceinline__ SyncArea resident_epoch(SyncArea s) {
   return s;
 }
 
-__device__ __forceinline__ int64_t flag_index(const Plan &p, int64_t n, int k, int t) {
-  return (n * p.nchunk + k) * p.tiles + t;
-}
-
 // 128-bit device-scope accesses through a raw buffer descriptor (cache policy sc1)
 constexpr int kAuxDeviceScope = 16;
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t record_buffer(const SyncArea &s) {
   return __builtin_amdgcn_make_buffer_rsrc(s.recs, 0, (int)s.rec_bytes, 0x27000);
+}
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t channel_record_buffer(const SyncArea &s) {
+  return __builtin_amdgcn_make_buffer_rsrc(s.crecs, 0, (int)s.crec_bytes, 0x27000);
 }
 __device__ __forceinline__ void record_store(__amdgpu_buffer_rsrc_t r, int64_t idx, float v0, float v1,
                                              unsigned long long epoch) {
@@ -151,36 +152,6 @@ __device__ __forceinline__ void for_group_records(const SyncArea &s, __amdgpu_bu
         body(__builtin_bit_cast(float, u0), __builtin_bit_cast(float, u1), record_count(p, tt[i], k_lo + kk[i], g));
       }
     }
-  }
-}
-
-// Every wave waits for the acknowledgement of its device-scope stores; after the workgroup barrier one
-// thread raises the workgroup's flag.
-__device__ __forceinline__ void publish_tile(const SyncArea &s, int64_t idx) {
-  __builtin_amdgcn_s_waitcnt(0);
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    __hip_atomic_store(&s.flags[idx], s.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-}
-
-// Wait until every (sample, row tile) workgroup of channel chunk k has raised its flag.
-__device__ __forceinline__ void wait_chunk_flags(const SyncArea &s, const Plan &p, int k) {
-  const int pairs = (int)p.N * p.tiles;
-  int spins = 0;
-  while (true) {
-    int ok = 1;
-    for (int e = threadIdx.x; e < pairs; e += kBlock) {
-      const int64_t nn = div_by(e, p.by_tiles);
-      const int t = e - (int)nn * p.tiles;
-      ok &= __hip_atomic_load(&s.flags[flag_index(p, nn, k, t)], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == s.epoch;
-    }
-    if (__syncthreads_and(ok)) break;
-    if (++spins > s.max_spins) {
-      if (threadIdx.x == 0) *s.status = s.epoch;
-      break;
-    }
-    __builtin_amdgcn_s_sleep(2);
   }
 }
 
@@ -312,13 +283,14 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 8 
 // ---------------------------------------------------------------------------------------------
 // Resident backward.  Same algebra as bwd_reduce_kernel + bwd_dx_kernel
 // (src/gnnhwc/csrc/gn_kernel.cu:598-618, 717-727, 783-800, 868-871), with x and dy read once.
-//   partC : [N][tiles][C][2]      records : {A, B, epoch} per (n, chunk, group, tile)
+//   group records   : {A, B, epoch} per (n, chunk, group, tile) of this launch
+//   channel records : {S1, S2, epoch} per (n, tile, channel) of the whole tensor (they feed dgamma / dbeta)
 // ---------------------------------------------------------------------------------------------
 template <typename T, typename PT, int VEC, int ACT, int NV>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 ? 4 : NV <= 8 ? 3 : NV <= 16 ? 2 : 1))) void fused_bwd_kernel(
     const T *__restrict__ x, const T *__restrict__ dy, T *__restrict__ dx, const void *mean, const void *rstd, int sdtype,
-    const void *w, const void *b, acc_t<T> *__restrict__ partC, SyncArea sync_arg, void *dw, void *db,
-    const acc_t<T> *partC_all, const void *mean_all, const void *rstd_all, int64_t n_all, Plan p) {
+    const void *w, const void *b, SyncArea sync_arg, void *dw, void *db, const void *mean_all, const void *rstd_all,
+    int64_t n0, int64_t n_all, Plan p) {
   using A = acc_t<T>;
   using LV = LaneVec<T, VEC>;
   const SyncArea sync = resident_epoch(sync_arg);
@@ -330,6 +302,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
   const int64_t n = blockIdx.z;
   const LanePos l = lane_pos(p, n, false);
   const __amdgpu_buffer_rsrc_t rb = record_buffer(sync);
+  const __amdgpu_buffer_rsrc_t rbc = channel_record_buffer(sync);
+  const void *safe = sync.recs;  // readable bytes for loads that only exist to keep the prologue free of branches
   const int rows = l.rows;
   const SafeLane sfl = safe_lane<VEC>(p, l, n);
   const int64_t off = sfl.off;
@@ -339,15 +313,15 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
   // the small loads go first: loads return in order, so the statistics and parameters, which the first row's
   // arithmetic needs, must not queue behind the whole tile.  Nothing here is under a branch (idle lanes read valid
   // addresses too), so every later wait counts exactly the loads it needs.
-  const StagedStats<A> st = fetch_chunk_stats<A>(mean, rstd, sdtype, p, l, sm_mu, sm_rs, partC);
+  const StagedStats<A> st = fetch_chunk_stats<A>(mean, rstd, sdtype, p, l, sm_mu, sm_rs, safe);
   A sa[VEC], sb[VEC], c1[VEC], c2[VEC];
-  lane_params_flat<A, PT, VEC>(sfl.c, w, b, partC, sa, sb);
+  lane_params_flat<A, PT, VEC>(sfl.c, w, b, safe, sa, sb);
   // gamma of the channel this thread handles when the tile's per-channel sums are published: fetched now, so that
   // the load is not part of the serial section between the sums and the record exchange
   A gamma0;
   {
     const int cg = (int)threadIdx.x < l.wch ? threadIdx.x : 0;
-    const PT *gp = w ? (const PT *)w + l.cstart + cg : (const PT *)partC;
+    const PT *gp = w ? (const PT *)w + l.cstart + cg : (const PT *)safe;
     const A gv = load_param<PT, A>(gp, 0);
     gamma0 = w ? gv : (A)1;
   }
@@ -390,9 +364,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
   }
   for (int c = threadIdx.x; c < l.wch; c += kBlock) {
     const A t1 = sm1[c], t2 = sm2[c];
-    const int64_t idx = ((n * p.tiles + l.tile) * p.C + l.cstart + c) * 2;
-    st_part<true>(partC + idx, t1);
-    st_part<true>(partC + idx + 1, t2);
+    record_store(rbc, ((n0 + n) * p.tiles + l.tile) * p.C + l.cstart + c, t1, t2, sync.epoch);
     const A gamma = c == (int)threadIdx.x ? gamma0 : (w ? load_param<PT, A>(w, l.cstart + c) : (A)1);
     sm1[c] = gamma * t1;
     sm2[c] = gamma * t2;
@@ -440,10 +412,35 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
       }
     }
   }
-  // partC went out before the records; by now those stores have long been acknowledged, so raising this tile's
-  // flag for the dgamma / dbeta workgroups costs no wait here (the barrier also orders the LDS writes above)
-  if (dw || db) publish_tile(sync, flag_index(p, n, l.chunk, l.tile));
-  else __syncthreads();
+  __syncthreads();
+  // dgamma / dbeta (compute_dweight_dbias, gn_kernel.cu:695-728).  The workgroups of this launch's first sample
+  // share the channels of their chunk: a segment of L lanes per channel sums the channel records of every
+  // (sample, row tile) pair of the whole tensor.  The records of this launch validate themselves by their epoch
+  // (no flags, no waiting for store acknowledgements anywhere); those of earlier launches over other groups of
+  // samples are complete because those launches have ended.  The first kTailFast records of a lane are requested
+  // here, so that their latency passes behind the dx phase below, and checked after it.
+  const bool tail = n == 0 && (dw || db);
+  const int pairs = (int)n_all * p.tiles;
+  const int TL = pow2_ceil_clamped(pairs, 64);
+  const int tlg = __builtin_ctz(TL);
+  const int cpp = kBlock >> tlg;  // channels per pass of the workgroup
+  const int tslot = threadIdx.x >> tlg, tsl = threadIdx.x & (TL - 1);
+  const bool tail_lane = tail && l.tile * cpp + tslot < l.wch;
+  const int tail_c = l.cstart + (tail_lane ? l.tile * cpp + tslot : 0);
+  const int tail_g = div_by(tail_c, p.by_D);
+  u32x4 trec[kTailFast];
+  A tmu[kTailFast], trs[kTailFast];
+  if (tail) {
+#pragma unroll
+    for (int i = 0; i < kTailFast; ++i) {
+      const int e = tsl + i * TL;
+      const int64_t nn = e < pairs ? e / p.tiles : 0;
+      const int t = e < pairs ? e - (int)nn * p.tiles : 0;
+      trec[i] = record_load(rbc, (nn * p.tiles + t) * p.C + tail_c);
+      tmu[i] = load_scalar_flat<A>(mean_all, nn * p.G + tail_g, sdtype, safe);
+      trs[i] = load_scalar_flat<A>(rstd_all, nn * p.G + tail_g, sdtype, safe);
+    }
+  }
   trace_point(sync, 3);
   if (rows > 0) {
     {
@@ -474,43 +471,51 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
     }
   }
   trace_point(sync, 4);
-  // dgamma / dbeta (compute_dweight_dbias, gn_kernel.cu:695-728): the workgroups of this launch's first sample
-  // share the channels of their chunk, a segment of L lanes per channel summing over every (sample, row tile)
-  // pair, once all tiles of this launch have published their per-channel sums.  The dx stores above drain
-  // meanwhile.  When the tensor is run as several launches over groups of samples only the last one gets dw / db;
-  // it sums over all n_all samples (partC_all, mean_all, rstd_all are the whole tensor's; the earlier launches
-  // have completed, so their sums need no flag).
-  if (n == 0 && (dw || db)) {
-    const int pairs = (int)n_all * p.tiles;
-    const int L = pow2_ceil_clamped(pairs, 64);
-    const int cpp = kBlock >> __builtin_ctz(L);  // channels per pass of the workgroup (L is a power of two)
-    const int slot = threadIdx.x >> __builtin_ctz(L), sl = threadIdx.x & (L - 1);
-    if (l.tile * cpp < l.wch) {
-      wait_chunk_flags(sync, p, l.chunk);
-      for (int cb = l.tile * cpp; cb < l.wch; cb += p.tiles * cpp) {
-        const int cc = cb + slot;
-        const bool valid = cc < l.wch;
-        const int c = l.cstart + cc;
-        A t1 = (A)0, t2 = (A)0;
-        if (valid) {
-          const int g = div_by(c, p.by_D);
-          for (int e = sl; e < pairs; e += L) {
-            const int64_t nn = e / p.tiles;
-            const int t = e - (int)nn * p.tiles;
-            const int64_t idx = ((nn * p.tiles + t) * p.C + c) * 2;
-            const A s1 = ld_part<true>(partC_all + idx);
-            const A s2 = ld_part<true>(partC_all + idx + 1);
-            const A mu = load_scalar<A>(mean_all, nn * p.G + g, sdtype);
-            const A rs = load_scalar<A>(rstd_all, nn * p.G + g, sdtype);
-            t1 += (s1 - mu * s2) * rs;
-            t2 += s2;
+  if (tail) {
+    int spins = 0;
+    for (int cb = l.tile * cpp; cb < l.wch; cb += p.tiles * cpp) {
+      const bool first = cb == l.tile * cpp;
+      const int cc = cb + tslot;
+      const bool valid = cc < l.wch;
+      const int c = l.cstart + (valid ? cc : 0);
+      const int g = div_by(c, p.by_D);
+      A t1 = (A)0, t2 = (A)0;
+      // one (sample, tile) pair: wait until its record is this launch's (if it is this launch's to write) and add it
+      auto add = [&](int e, u32x4 rec, A mu, A rs) {
+        const int64_t nn = e / p.tiles;
+        const int t = e - (int)nn * p.tiles;
+        while (valid && nn >= n0 && !record_ready(rec, sync.epoch)) {
+          if (++spins > sync.max_spins) {
+            *sync.status = sync.epoch;
+            break;
           }
+          __builtin_amdgcn_s_sleep(2);
+          rec = record_load(rbc, (nn * p.tiles + t) * p.C + c);
         }
-        segment_sum2(t1, t2, L);
-        if (valid && sl == 0) {
-          if (dw) store_param<PT, A>(dw, c, t1);
-          if (db) store_param<PT, A>(db, c, t2);
+        const unsigned u0 = rec.x, u1 = rec.y;
+        const A s1 = __builtin_bit_cast(float, u0), s2 = __builtin_bit_cast(float, u1);
+        t1 += (s1 - mu * s2) * rs;
+        t2 += s2;
+      };
+      int e = tsl;
+      if (first) {  // the records requested before the dx phase
+#pragma unroll
+        for (int i = 0; i < kTailFast; ++i) {
+          if (e < pairs) add(e, trec[i], tmu[i], trs[i]);
+          e += TL;
         }
+      }
+      for (; e < pairs; e += TL) {
+        const int64_t nn = e / p.tiles;
+        const int t = e - (int)nn * p.tiles;
+        add(e, record_load(rbc, (nn * p.tiles + t) * p.C + c), load_scalar<A>(mean_all, nn * p.G + g, sdtype),
+            load_scalar<A>(rstd_all, nn * p.G + g, sdtype));
+      }
+      if (!valid) { t1 = (A)0; t2 = (A)0; }
+      segment_sum2(t1, t2, TL);
+      if (valid && tsl == 0) {
+        if (dw) store_param<PT, A>(dw, c, t1);
+        if (db) store_param<PT, A>(db, c, t2);
       }
     }
     trace_point(sync, 5);

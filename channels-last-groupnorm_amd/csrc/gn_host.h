@@ -76,16 +76,15 @@ inline size_t resident_fwd_bytes(int64_t G) { return kWorkspaceHeader + align_up
 // A tensor of several samples that is too large for one single-launch kernel may still be run as up to
 // kMaxBatches such launches over consecutive groups of samples (samples share nothing but dgamma / dbeta).
 constexpr int kMaxBatches = 4;
-// Per-channel tile sums of the backward, [N][tiles][C][2] floats: one launch's worth at most
-// 2 * chunk_channels * kMaxResidentBlocks, and room for the launches of a batched call up to a fixed bound.
-inline size_t resident_partc_bytes(int64_t chunk_channels) {
-  const size_t one = (size_t)2 * chunk_channels * kMaxResidentBlocks * 4;
-  const size_t many = one * kMaxBatches < ((size_t)8 << 20) ? one * kMaxBatches : ((size_t)8 << 20);
+// Channel records of the backward, 16 bytes per (sample, tile, channel): one launch's worth is at most
+// chunk_channels * kMaxResidentBlocks of them, and there is room for the launches of a batched call up to a bound.
+inline size_t resident_crec_bytes(int64_t chunk_channels) {
+  const size_t one = (size_t)16 * chunk_channels * kMaxResidentBlocks;
+  const size_t many = one * kMaxBatches < ((size_t)16 << 20) ? one * kMaxBatches : ((size_t)16 << 20);
   return align_up(one > many ? one : many, 256);
 }
 inline size_t resident_bwd_bytes(int64_t chunk_channels, int64_t G) {
-  return kWorkspaceHeader + resident_partc_bytes(chunk_channels) + align_up(resident_rec_bytes(G), 256) +
-         (size_t)kMaxResidentBlocks * 8;
+  return kWorkspaceHeader + resident_crec_bytes(chunk_channels) + align_up(resident_rec_bytes(G), 256);
 }
 // A fresh nonzero 64-bit value per call (gn_api.hip).
 unsigned long long next_epoch();

@@ -91,7 +91,6 @@ bool resident_tiling(const Plan &base, int64_t samples, int nv, int slots, Plan 
 }
 
 struct ResidentWorkspace {
-  A *partC;  // backward only
   SyncArea sync;
   unsigned long long *generation;  // device word in the workspace header
 };
@@ -115,10 +114,10 @@ void arm_generation(ResidentWorkspace &r, hipStream_t stream) {
 ResidentWorkspace resident_fwd_ws(void *ws, const Plan &p) {
   ResidentWorkspace r;
   char *base = (char *)ws + kWorkspaceHeader;
-  r.partC = nullptr;
   r.sync.recs = base;
   r.sync.rec_bytes = (unsigned)resident_rec_bytes(p.G);
-  r.sync.flags = nullptr;
+  r.sync.crecs = nullptr;
+  r.sync.crec_bytes = 0;
   r.sync.status = resident_status();
   r.generation = (unsigned long long *)ws;
   r.sync.max_spins = resident_spin_limit();
@@ -131,12 +130,10 @@ ResidentWorkspace resident_bwd_ws(void *ws, const Plan &p) {
   ResidentWorkspace r;
   char *base = (char *)ws + kWorkspaceHeader;
   const size_t cc = (size_t)p.lpr * p.vec;
-  r.partC = (A *)base;
-  char *recs = base + resident_partc_bytes(cc);
-  r.sync.recs = recs;
+  r.sync.crecs = base;  // channel records of the whole tensor, [N][tiles][C] x 16 bytes
+  r.sync.crec_bytes = (unsigned)resident_crec_bytes(cc);
+  r.sync.recs = base + resident_crec_bytes(cc);
   r.sync.rec_bytes = (unsigned)resident_rec_bytes(p.G);
-  char *f = recs + align_up(resident_rec_bytes(p.G), 256);
-  r.sync.flags = (unsigned long long *)f;
   r.sync.status = resident_status();
   r.generation = (unsigned long long *)ws;
   r.sync.max_spins = resident_spin_limit();
@@ -211,9 +208,9 @@ template <typename PT, int ACT, int NV> bool try_resident_bwd_nv(const BwdArgs &
   const int64_t per = (a.plan.N + batches - 1) / batches;
   Plan p;
   if (!resident_tiling(a.plan, per, NV, slots, p)) return false;
-  // per-channel tile sums of every sample stay in the workspace until the last launch has summed them
-  const size_t partc_need = (size_t)a.plan.N * p.tiles * a.plan.C * 2 * sizeof(A);
-  if (partc_need > resident_partc_bytes((int64_t)p.lpr * p.vec)) return false;
+  // the channel records of every sample stay in the workspace until the last launch has summed them
+  const size_t crec_need = (size_t)a.plan.N * p.tiles * a.plan.C * 16;
+  if (crec_need > resident_crec_bytes((int64_t)p.lpr * p.vec)) return false;
   if (!resident_status()) return false;
   mark_resident_launch();
   const int64_t sample = a.plan.R * a.plan.C;
@@ -225,11 +222,10 @@ template <typename PT, int ACT, int NV> bool try_resident_bwd_nv(const BwdArgs &
     ResidentWorkspace r = resident_bwd_ws(a.ws, pb);
     arm_generation(r, a.stream);
     const bool last = n0 + per >= a.plan.N;
-    A *partC_here = r.partC + n0 * p.tiles * a.plan.C * 2;
     launch(kKindFusedBwd, kernel, tile_grid(pb, 0), dim3(kBlock), a.stream, (const elem_t *)a.x + n0 * sample,
            (const elem_t *)a.dy + n0 * sample, (elem_t *)a.dx + n0 * sample, (const char *)a.mean + n0 * a.plan.G * ssz,
-           (const char *)a.rstd + n0 * a.plan.G * ssz, a.sdtype, a.w, a.b, partC_here, r.sync, last ? a.dw : nullptr,
-           last ? a.db : nullptr, (const A *)r.partC, a.mean, a.rstd, a.plan.N, pb);
+           (const char *)a.rstd + n0 * a.plan.G * ssz, a.sdtype, a.w, a.b, r.sync, last ? a.dw : nullptr,
+           last ? a.db : nullptr, a.mean, a.rstd, n0, a.plan.N, pb);
   }
   return true;
 }
