@@ -21,3 +21,13 @@ def device():
     if not torch.cuda.is_available():
         pytest.skip("no GPU visible")
     return torch.device("cuda:0")
+
+
+@pytest.fixture(params=["resident", "streaming"])
+def family(request):
+    """Runs a GPU test once with the single-launch kernels allowed and once with the streaming kernels only."""
+    from gnnhwc import _cabi
+
+    before = _cabi.set_resident(request.param == "resident")
+    yield request.param
+    _cabi.set_resident(before)

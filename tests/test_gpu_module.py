@@ -22,13 +22,6 @@ TOL = {torch.float32: 1e-5, torch.float64: 1e-12}
 HALF_SLACK = 0.02
 
 
-@pytest.fixture(params=["resident", "streaming"])
-def family(request):
-    before = _cabi.set_resident(request.param == "resident")
-    yield request.param
-    _cabi.set_resident(before)
-
-
 def channels_last_like(shape, dtype, device, gen, scale=1.0, shift=0.0):
     """Random (N, C, *spatial) tensor whose memory is (N, *spatial, C): stride(1) == 1 for any rank."""
     N, C = shape[0], shape[1]

@@ -64,7 +64,7 @@ def _check(name, ours, truth, lib_result, dtype, mask=None):
 
 
 @pytest.mark.parametrize("name", configs.ALL_NAMES)
-def test_config_parity(name, device):
+def test_config_parity(family, name, device):
     cfg = configs.CONFIGS[name]
     print("config", name, cfg, flush=True)
     inp = configs.make_inputs(cfg, device)
