@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused NHWC GroupNorm + activation forward / backward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload sd_unet|<config name>] [--all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload sd_unet|all|<config name>] [--all]
 
 A "step" is one forward + backward call of the op, through the C ABI of libgnnhwc_hip.so, on each shape
 of the workload (default: the latent-diffusion UNet sweep c3a, c3b, c3c in bf16 with fused SiLU), with
@@ -349,7 +349,12 @@ def main():
     torch.cuda.set_device(device)
     use_graph = args.graph
 
-    head_names = list(configs.SD_UNET_SWEEP) if args.workload == "sd_unet" else [args.workload]
+    if args.workload == "sd_unet":
+        head_names = list(configs.SD_UNET_SWEEP)
+    elif args.workload == "all":
+        head_names = list(configs.ALL_NAMES)
+    else:
+        head_names = [args.workload]
     probs = [Problem(configs.CONFIGS[n], device) for n in head_names]
     stream_of = lambda: torch.cuda.current_stream().cuda_stream  # noqa: E731
 
@@ -421,7 +426,8 @@ def main():
         torch.cuda.empty_cache()
 
     line = {
-        "metric": "fused GN+SiLU fwd+bwd achieved HBM GB/s (algorithmic bytes / time), SD-UNet shapes",
+        "metric": ("fused GN+SiLU fwd+bwd achieved HBM GB/s (algorithmic bytes / time), SD-UNet shapes" if args.workload == "sd_unet"
+                   else "fused GN+activation achieved HBM GB/s (algorithmic bytes / time), workload %s" % args.workload),
         "value": round(value, 1),
         "unit": "GB/s",
         "n_gpus": 1,
@@ -433,9 +439,12 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": {"bf16": "bf16 data, f32 arithmetic", "fp16": "f16 data, f32 arithmetic", "fp32": "f32", "fp64": "f64"}[probs[0].cfg.dtype],
+        "dtype": ({"bf16": "bf16 data, f32 arithmetic", "fp16": "f16 data, f32 arithmetic", "fp32": "f32", "fp64": "f64"}[probs[0].cfg.dtype]
+                  if len({p.cfg.dtype for p in probs}) == 1 else "mixed (f32 arithmetic)"),
         "data": "synthetic (seeded)",
-        "config": {"workload": "+".join(head_names), "passes": "fwd+bwd", "activation": probs[0].cfg.act,
+        "config": {"workload": "+".join(head_names) if len(head_names) <= 4 else "%s (%d configurations)" % (args.workload, len(head_names)),
+                   "passes": "fwd+bwd" if all(p.bwd for p in probs) else "per configuration",
+                   "activation": probs[0].cfg.act if len({p.cfg.act for p in probs}) == 1 else "per configuration",
                    "timing": "HIP graph replay of the K steps" if use_graph else "eager launches through the C ABI",
                    "algorithmic_bytes_per_step": alg},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
