@@ -214,6 +214,9 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 8 
   }
   const __amdgpu_buffer_rsrc_t rb = record_buffer(sync);
   trace_point(sync, 1, (float)m2[0]);
+  // the reduction and the exchange are one chain of dependent steps that every workgroup of the group waits for:
+  // let these wavefronts go first on a SIMD they share with wavefronts of other workgroups that are still streaming
+  __builtin_amdgcn_s_setprio(3);
   block_group_moments<A, VEC>(p, l, mean, m2, sm0, sm1, [&](int g, A cnt, A mu, A s2) {
     (void)cnt;  // the consumers recompute it from the geometry
     record_store(rb, group_slot(q, p.G, n, l.tile, l.chunk, g), mu, s2, sync.epoch);
@@ -261,6 +264,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 8 
     }
     __syncthreads();
   }
+  __builtin_amdgcn_s_setprio(0);
   trace_point(sync, 3);
   if (rows > 0) {
     A unused1[VEC], unused2[VEC];
@@ -360,6 +364,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
       }
     }
     trace_point(sync, 6, (float)(s1[0] + s2[0]));
+    __builtin_amdgcn_s_setprio(3);  // as in the forward: the serial chain to the exchange goes first
     block_channel_sums<A, VEC>(p, l, s1, s2, sm1, sm2);
   }
   for (int c = threadIdx.x; c < l.wch; c += kBlock) {
@@ -419,6 +424,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
   // (no flags, no waiting for store acknowledgements anywhere); those of earlier launches over other groups of
   // samples are complete because those launches have ended.  The first kTailFast records of a lane are requested
   // here, so that their latency passes behind the dx phase below, and checked after it.
+  __builtin_amdgcn_s_setprio(0);
   const bool tail = n == 0 && (dw || db);
   const int pairs = (int)n_all * p.tiles;
   const int TL = pow2_ceil_clamped(pairs, 64);
