@@ -187,6 +187,9 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 8 
   }
   A sa[VEC], sb[VEC];
   if (rows > 0) lane_params<A, PT, VEC>(l, w, b, sa, sb);  // needed after the exchange; in flight until then
+  // everything up to the exchange is on the critical path of the whole group; what follows it is not: a wavefront
+  // still working towards the exchange goes before one (of another workgroup on the same SIMD) that is past it
+  __builtin_amdgcn_s_setprio(2);
   A mean[VEC], m2[VEC];
 #pragma unroll
   for (int j = 0; j < VEC; ++j) { mean[j] = (A)0; m2[j] = (A)0; }
@@ -337,6 +340,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
     bd[u] = LV::load(dy + o);
   }
   commit_chunk_stats<A>(st, l, sm_mu, sm_rs);
+  __builtin_amdgcn_s_setprio(2);  // towards the exchange: ahead of wavefronts that are already past theirs
   __syncthreads();
   trace_point(sync, 1);
   {
