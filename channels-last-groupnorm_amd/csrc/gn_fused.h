@@ -349,22 +349,40 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
     for (int j = 0; j < VEC; ++j) { s1[j] = (A)0; s2[j] = (A)0; }
     if (rows > 0) {
       lane_coeffs<A, VEC, false>(p, l, sm_mu, sm_rs, nullptr, nullptr, sa, sb, c1, c2);
+      // dy is not needed again: its registers keep g' = dy * act'(z) for the dx phase (for 16-bit data
+      // rounded to T, the rounding an unfused activation backward applies to the same quantity).
+      // A full tile (all but the last tile of a sample) needs no masking of rows past the lane's last one.
+      if (rows == NV) {
 #pragma unroll
-      for (int u = 0; u < NV; ++u) {
-        const A keep = u < rows ? (A)1 : (A)0;
-        A vx[VEC], vd[VEC];
-        LV::unpack(bx[u], vx);
-        LV::unpack(bd[u], vd);
+        for (int u = 0; u < NV; ++u) {
+          A vx[VEC], vd[VEC];
+          LV::unpack(bx[u], vx);
+          LV::unpack(bd[u], vd);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) {
-          const A g = keep * vd[j] * act_bwd<ACT, A>(vx[j] * sa[j] + sb[j]);
-          s1[j] += g * vx[j];
-          s2[j] += g;
-          vd[j] = g;
+          for (int j = 0; j < VEC; ++j) {
+            const A g = vd[j] * act_bwd<ACT, A>(vx[j] * sa[j] + sb[j]);
+            s1[j] += g * vx[j];
+            s2[j] += g;
+            vd[j] = g;
+          }
+          bd[u] = LV::pack(vd);
         }
-        // dy is not needed again: its registers keep g' = dy * act'(z) for the dx phase (for 16-bit data
-        // rounded to T, the rounding an unfused activation backward applies to the same quantity)
-        bd[u] = LV::pack(vd);
+      } else {
+#pragma unroll
+        for (int u = 0; u < NV; ++u) {
+          const A keep = u < rows ? (A)1 : (A)0;
+          A vx[VEC], vd[VEC];
+          LV::unpack(bx[u], vx);
+          LV::unpack(bd[u], vd);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) {
+            const A g = keep * vd[j] * act_bwd<ACT, A>(vx[j] * sa[j] + sb[j]);
+            s1[j] += g * vx[j];
+            s2[j] += g;
+            vd[j] = g;
+          }
+          bd[u] = LV::pack(vd);
+        }
       }
     }
     trace_point(sync, 6, (float)(s1[0] + s2[0]));
