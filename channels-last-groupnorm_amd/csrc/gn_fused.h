@@ -30,7 +30,7 @@
 namespace gn {
 
 constexpr int kMaxSpins = 1 << 22;  // default bound on the polls of one wait (seconds of polling)
-constexpr int kRecFast = 4;
+constexpr int kRecFast = 2;
 constexpr int kTailFast = 2;  // channel records a lane of the dgamma / dbeta stage requests ahead of the dx phase
 constexpr int kMaxResidentBlocksDev = 4 * kNumCU;  // records a lane keeps in registers while polling
 
