@@ -179,14 +179,21 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 8 
   const int64_t step = (int64_t)p.rpi * p.C;
   typename LV::raw_t buf[NV];
   trace_point(sync, 0);
+  // gamma / beta are needed only after the exchange, but they are requested first and without any branch: a load
+  // under a branch makes the compiler drain every outstanding load where the branch joins, and then the statistics
+  // below could not start on the first rows while the later ones are still arriving
+  A sa[VEC], sb[VEC];
+  {
+    const int cvi = l.cvi < p.cv ? l.cvi : p.cv - 1;
+    lane_params_flat<A, PT, VEC>(cvi * VEC, w, b, sync.recs, sa, sb);
+  }
+  issue_order_fence();
   if (rows > 0) {
     // every load is unconditional (rows past the lane's last one re-read it): the waits that follow can then
     // count loads exactly, and row u is processed while rows u + 1 ... are still in flight
 #pragma unroll
     for (int u = 0; u < NV; ++u) buf[u] = LV::load(x + off + (int64_t)clamp_row(u, rows) * step);
   }
-  A sa[VEC], sb[VEC];
-  if (rows > 0) lane_params<A, PT, VEC>(l, w, b, sa, sb);  // needed after the exchange; in flight until then
   // everything up to the exchange is on the critical path of the whole group; what follows it is not: a wavefront
   // still working towards the exchange goes before one (of another workgroup on the same SIMD) that is past it
   __builtin_amdgcn_s_setprio(2);
