@@ -186,6 +186,13 @@ template <typename ACC> __device__ __forceinline__ void store_scalar(void *p, in
 // ---------------------------------------------------------------------------------------------
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 __device__ __forceinline__ double fast_rcp(double x) { return 1.0 / x; }
+// 1 / sqrt(v): hardware estimate (1 ulp) refined by one Newton step; a few instructions where the division
+// sequence takes a dozen, and these sit in the serial section every workgroup of a group waits for.
+__device__ __forceinline__ float fast_rsqrt(float v) {
+  const float r = __builtin_amdgcn_rsqf(v);
+  return r * (1.5f - 0.5f * v * r * r);
+}
+__device__ __forceinline__ double fast_rsqrt(double v) { return 1.0 / sqrt(v); }
 // logistic sigmoid 1/(1+e^-x); exp2 overflow to +inf gives rcp(inf) = 0, underflow gives 1.
 __device__ __forceinline__ float sigmoid(float x) {
   return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.44269504088896340736f));

@@ -252,7 +252,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 8 
         s1 += cnt * d;
         s2 += mm + cnt * d * d;
       });
-      const A inv = nl > (A)0 ? (A)1 / nl : (A)0;
+      const A inv = nl > (A)0 ? fast_rcp(nl) : (A)0;
       const A mean_l = kl + s1 * inv;
       const A m2_l = s2 - s1 * s1 * inv;
       // ... and the lanes are merged about the first lane's mean
@@ -261,9 +261,9 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 8 
       A t1 = nl * d, t2 = m2_l + nl * d * d;
       segment_sum2(t1, t2, L);
       if (valid && sl == 0) {
-        const A dm = t1 / total;
+        const A dm = t1 * fast_rcp(total);
         const A gmean = K + dm;
-        const A rs = (A)1 / sqrt((t2 - t1 * dm) / total + eps);
+        const A rs = fast_rsqrt((t2 - t1 * dm) * fast_rcp(total) + eps);
         sm0[gi] = gmean;
         sm1[gi] = rs;
         if (l.tile == 0 && g * p.D >= l.cstart) {
@@ -396,10 +396,19 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
     __builtin_amdgcn_s_setprio(3);  // as in the forward: the serial chain to the exchange goes first
     block_channel_sums<A, VEC>(p, l, s1, s2, sm1, sm2);
   }
-  for (int c = threadIdx.x; c < l.wch; c += kBlock) {
+  // publish the tile's per-channel sums and keep gamma-weighted copies for the group sums; the first channel of a
+  // thread uses the gamma fetched in the prologue (no load in this serial section), wider chunks load the rest
+  if ((int)threadIdx.x < l.wch) {
+    const int c = threadIdx.x;
     const A t1 = sm1[c], t2 = sm2[c];
     record_store(rbc, ((n0 + n) * p.tiles + l.tile) * p.C + l.cstart + c, t1, t2, sync.epoch);
-    const A gamma = c == (int)threadIdx.x ? gamma0 : (w ? load_param<PT, A>(w, l.cstart + c) : (A)1);
+    sm1[c] = gamma0 * t1;
+    sm2[c] = gamma0 * t2;
+  }
+  for (int c = threadIdx.x + kBlock; c < l.wch; c += kBlock) {
+    const A t1 = sm1[c], t2 = sm2[c];
+    record_store(rbc, ((n0 + n) * p.tiles + l.tile) * p.C + l.cstart + c, t1, t2, sync.epoch);
+    const A gamma = w ? load_param<PT, A>(w, l.cstart + c) : (A)1;
     sm1[c] = gamma * t1;
     sm2[c] = gamma * t2;
   }
@@ -439,7 +448,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
       if (valid && sl == 0) {
         const A mu = sm_mu[gi];
         const A rs = sm_rs[gi];
-        const A s = (A)1 / ((A)p.D * (A)p.R);
+        const A s = fast_rcp((A)p.D * (A)p.R);
         const A k1 = (mu * tb - ta) * s * rs * rs * rs;
         sm1[gi] = k1;
         sm2[gi] = -mu * k1 - tb * s * rs;

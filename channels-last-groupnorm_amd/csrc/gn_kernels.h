@@ -196,7 +196,7 @@ template <typename A> __device__ __forceinline__ Moments<A> reduce_moments(const
     s1 += cn * d;
     s2 += (h ? e.v[i][2] : (A)0) + cn * d * d;
   }
-  const A inv = nl > (A)0 ? (A)1 / nl : (A)0;
+  const A inv = nl > (A)0 ? fast_rcp(nl) : (A)0;
   const A mean_l = kl + s1 * inv;
   const A m2_l = s2 - s1 * s1 * inv;
   const A K = __shfl(mean_l, (int)(threadIdx.x & 63 & ~(e.L - 1)), 64);
@@ -206,7 +206,7 @@ template <typename A> __device__ __forceinline__ Moments<A> reduce_moments(const
   segment_sum2(t1, t2, e.L);
   Moments<A> r;
   r.n = t0;
-  const A dm = e.valid ? t1 / t0 : (A)0;
+  const A dm = e.valid ? t1 * fast_rcp(t0) : (A)0;
   r.mean = K + dm;
   r.m2 = t2 - t1 * dm;
   return r;
@@ -379,7 +379,7 @@ __device__ __forceinline__ void block_group_moments(const Plan &p, const LanePos
     segment_sum2(s1, s2, L);
     if (valid && sl == 0) {
       const A total = (A)(cb - ca) * nrows;
-      const A dm = s1 / total;
+      const A dm = s1 * fast_rcp(total);
       emit(g, total, K + dm, s2 - s1 * dm);
     }
   }
@@ -462,7 +462,7 @@ __device__ __forceinline__ Moments<A> merge_group_partials(const A *__restrict__
     s1 += cn * d;
     s2 += mm + cn * d * d;
   }
-  const A inv = nl > (A)0 ? (A)1 / nl : (A)0;
+  const A inv = nl > (A)0 ? fast_rcp(nl) : (A)0;
   const A mean_l = kl + s1 * inv;
   const A m2_l = s2 - s1 * s1 * inv;
   const A K = __shfl(mean_l, (int)(threadIdx.x & 63 & ~(L - 1)), 64);
@@ -472,7 +472,7 @@ __device__ __forceinline__ Moments<A> merge_group_partials(const A *__restrict__
   segment_sum2(t1, t2, L);
   Moments<A> r;
   r.n = t0;
-  const A dm = valid ? t1 / t0 : (A)0;
+  const A dm = valid ? t1 * fast_rcp(t0) : (A)0;
   r.mean = K + dm;
   r.m2 = t2 - t1 * dm;
   return r;
@@ -517,7 +517,7 @@ __device__ __forceinline__ void merge_chunk_stats(const A *__restrict__ part, co
     const int g = l.g_lo + gi;
     const Moments<A> m = merge_group_partials<A, COH>(part, plane, q, p.G, p.D, l.n, g, valid, L, sl);
     if (valid && sl == 0) {
-      const A rs = (A)1 / sqrt(m.m2 / m.n + eps);
+      const A rs = fast_rsqrt(m.m2 * fast_rcp(m.n) + eps);
       sm_mu[gi] = m.mean;
       sm_rs[gi] = rs;
       if (l.tile == 0 && g * p.D >= l.cstart) {  // the chunk where the group starts reports it
@@ -692,7 +692,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
       const Moments<A> m = reduce_moments<A>(early);
       if (early.valid && early.sl == 0) {
         const int g = l.g_lo + early.gi;
-        const A rs = (A)1 / sqrt(m.m2 / m.n + eps);
+        const A rs = fast_rsqrt(m.m2 * fast_rcp(m.n) + eps);
         sm_mu[early.gi] = m.mean;
         sm_rs[early.gi] = rs;
         if (l.tile == 0 && g * p.D >= l.cstart) {  // the chunk where the group starts reports it
@@ -787,12 +787,22 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
     }
     block_channel_sums<A, VEC>(p, l, s1, s2, sm1, sm2);
     // per channel: publish the tile sums; keep gamma-weighted copies for the group sums
-    for (int c = threadIdx.x; c < l.wch; c += kBlock) {
+    // (a thread's first channel uses the gamma fetched in the prologue: no load in this serial tail)
+    if ((int)threadIdx.x < l.wch) {
+      const int c = threadIdx.x;
       const A t1 = sm1[c], t2 = sm2[c];
       const int64_t idx = ((n * p.tiles + l.tile) * p.C + l.cstart + c) * 2;
       partC[idx] = t1;
       partC[idx + 1] = t2;
-      const A gamma = c == (int)threadIdx.x ? gamma0 : (w ? load_param<PT, A>(w, l.cstart + c) : (A)1);
+      sm1[c] = gamma0 * t1;
+      sm2[c] = gamma0 * t2;
+    }
+    for (int c = threadIdx.x + kBlock; c < l.wch; c += kBlock) {
+      const A t1 = sm1[c], t2 = sm2[c];
+      const int64_t idx = ((n * p.tiles + l.tile) * p.C + l.cstart + c) * 2;
+      partC[idx] = t1;
+      partC[idx + 1] = t2;
+      const A gamma = w ? load_param<PT, A>(w, l.cstart + c) : (A)1;
       sm1[c] = gamma * t1;
       sm2[c] = gamma * t2;
     }
@@ -1018,7 +1028,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
       A ta, tb;
       reduce_sums<A>(early, ta, tb);
       if (early.valid && early.sl == 0) {
-        const A s = (A)1 / ((A)p.D * (A)p.R);
+        const A s = fast_rcp((A)p.D * (A)p.R);
         const A k1 = (emu * tb - ta) * s * ers * ers * ers;
         sm_mu[early.gi] = emu;
         sm_rs[early.gi] = ers;
@@ -1038,7 +1048,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
         if (valid && sl == 0) {
           const A mu = load_scalar<A>(mean, n * p.G + g, sdtype);
           const A rs = load_scalar<A>(rstd, n * p.G + g, sdtype);
-          const A s = (A)1 / ((A)p.D * (A)p.R);
+          const A s = fast_rcp((A)p.D * (A)p.R);
           const A k1 = (mu * tb - ta) * s * rs * rs * rs;
           sm_mu[gi] = mu;
           sm_rs[gi] = rs;
