@@ -95,14 +95,21 @@ __device__ __forceinline__ bool record_ready(const u32x4 &rec, unsigned long lon
 }
 
 // Elements behind record (tile t, chunk k, group g): the rows of the tile times the channels of g in chunk k.
+// (32-bit arithmetic: channel indices and the rows of a tile fit, and 64-bit multiplies are slow here)
 __device__ __forceinline__ float record_count(const Plan &p, int t, int k, int g) {
   const int cc = p.lpr * p.vec;
-  const int64_t c_lo = (int64_t)g * p.D > (int64_t)k * cc ? (int64_t)g * p.D : (int64_t)k * cc;
-  int64_t c_hi = (int64_t)(g + 1) * p.D < (int64_t)(k + 1) * cc ? (int64_t)(g + 1) * p.D : (int64_t)(k + 1) * cc;
-  if (c_hi > p.C) c_hi = p.C;
-  const int64_t rem = p.R - (int64_t)t * p.tile_rows;
-  const int64_t rows = rem < p.tile_rows ? rem : p.tile_rows;
-  return (float)((c_hi - c_lo) * rows);
+  const int c_lo = g * p.D > k * cc ? g * p.D : k * cc;
+  int c_hi = (g + 1) * p.D < (k + 1) * cc ? (g + 1) * p.D : (k + 1) * cc;
+  if (c_hi > (int)p.C) c_hi = (int)p.C;
+  const int64_t rem = p.R - (int64_t)t * p.tile_rows;  // t * tile_rows: one 32 x 32 -> 64 multiply
+  const int rows = rem < p.tile_rows ? (int)rem : p.tile_rows;
+  return (float)(c_hi - c_lo) * (float)rows;
+}
+// Slot of a record, in 32 bits with 24-bit multiplies: a single-launch kernel has at most kMaxResidentBlocksDev
+// workgroups, so (n nchunk + k) and tiles are small, and the host only sizes the record area for G below 2^20.
+__device__ __forceinline__ int record_slot(const PartialGeo &q, int G, int n, int t, int k, int g) {
+  const int col = __mul24(n, q.nchunk) + k;
+  return __mul24(__mul24(col, G) + g, q.tiles) + t;
 }
 
 // Collect the records of group g (all tiles of the chunks that hold a piece of it) with L lanes and reduce
@@ -115,13 +122,13 @@ __device__ __forceinline__ void for_group_records(const SyncArea &s, __amdgpu_bu
   int k_lo = 0, nk = 1;
   if (valid) group_chunks(q, p.D, g, k_lo, nk);
   const int P = valid ? q.tiles * nk : 0;
-  const int64_t base = group_slot(q, p.G, n, 0, k_lo, g);
-  const int64_t kstride = (int64_t)p.G * q.tiles;
+  const int base = record_slot(q, p.G, (int)n, 0, k_lo, g);
+  const int kstride = __mul24(p.G, q.tiles);
   int spins = 0;
   for (int e0 = sl; e0 < P; e0 += kRecFast * L) {
     u32x4 rec[kRecFast];
     bool have[kRecFast];
-    int64_t idx[kRecFast];
+    int idx[kRecFast];
     int kk[kRecFast], tt[kRecFast];
 #pragma unroll
     for (int i = 0; i < kRecFast; ++i) {
@@ -129,7 +136,7 @@ __device__ __forceinline__ void for_group_records(const SyncArea &s, __amdgpu_bu
       have[i] = e < P;
       kk[i] = have[i] ? div_by(e, q.by_tiles) : 0;
       tt[i] = have[i] ? e - kk[i] * q.tiles : 0;
-      idx[i] = base + kk[i] * kstride + tt[i];
+      idx[i] = base + __mul24(kk[i], kstride) + tt[i];
     }
     while (true) {
       bool ok = true;
@@ -229,7 +236,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 8 
   __builtin_amdgcn_s_setprio(3);
   block_group_moments<A, VEC>(p, l, mean, m2, sm0, sm1, [&](int g, A cnt, A mu, A s2) {
     (void)cnt;  // the consumers recompute it from the geometry
-    record_store(rb, group_slot(q, p.G, n, l.tile, l.chunk, g), mu, s2, sync.epoch);
+    record_store(rb, record_slot(q, p.G, (int)n, l.tile, l.chunk, g), mu, s2, sync.epoch);
   });
   trace_point(sync, 2);
   {
@@ -396,18 +403,20 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
     __builtin_amdgcn_s_setprio(3);  // as in the forward: the serial chain to the exchange goes first
     block_channel_sums<A, VEC>(p, l, s1, s2, sm1, sm2);
   }
+  // (channel records are indexed in 32 bits: their area is a few megabytes)
+  const int crec_row = __mul24(__mul24((int)(n0 + n), p.tiles) + l.tile, (int)p.C) + l.cstart;
   // publish the tile's per-channel sums and keep gamma-weighted copies for the group sums; the first channel of a
   // thread uses the gamma fetched in the prologue (no load in this serial section), wider chunks load the rest
   if ((int)threadIdx.x < l.wch) {
     const int c = threadIdx.x;
     const A t1 = sm1[c], t2 = sm2[c];
-    record_store(rbc, ((n0 + n) * p.tiles + l.tile) * p.C + l.cstart + c, t1, t2, sync.epoch);
+    record_store(rbc, crec_row + c, t1, t2, sync.epoch);
     sm1[c] = gamma0 * t1;
     sm2[c] = gamma0 * t2;
   }
   for (int c = threadIdx.x + kBlock; c < l.wch; c += kBlock) {
     const A t1 = sm1[c], t2 = sm2[c];
-    record_store(rbc, ((n0 + n) * p.tiles + l.tile) * p.C + l.cstart + c, t1, t2, sync.epoch);
+    record_store(rbc, crec_row + c, t1, t2, sync.epoch);
     const A gamma = w ? load_param<PT, A>(w, l.cstart + c) : (A)1;
     sm1[c] = gamma * t1;
     sm2[c] = gamma * t2;
@@ -426,7 +435,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
       A ta = (A)0, tb = (A)0;
       for (int c = ca + sl; c < cb; c += L) { ta += sm1[c]; tb += sm2[c]; }
       segment_sum2(ta, tb, L);
-      if (valid && sl == 0) record_store(rb, group_slot(q, p.G, n, l.tile, l.chunk, g), ta, tb, sync.epoch);
+      if (valid && sl == 0) record_store(rb, record_slot(q, p.G, (int)n, l.tile, l.chunk, g), ta, tb, sync.epoch);
     }
   }
   __syncthreads();
@@ -478,9 +487,9 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
 #pragma unroll
     for (int i = 0; i < kTailFast; ++i) {
       const int e = tsl + i * TL;
-      const int64_t nn = e < pairs ? e / p.tiles : 0;
-      const int t = e < pairs ? e - (int)nn * p.tiles : 0;
-      trec[i] = record_load(rbc, (nn * p.tiles + t) * p.C + tail_c);
+      const int nn = e < pairs ? e / p.tiles : 0;
+      const int t = e < pairs ? e - nn * p.tiles : 0;
+      trec[i] = record_load(rbc, __mul24(__mul24(nn, p.tiles) + t, (int)p.C) + tail_c);
       tmu[i] = load_scalar_flat<A>(mean_all, nn * p.G + tail_g, sdtype, safe);
       trs[i] = load_scalar_flat<A>(rstd_all, nn * p.G + tail_g, sdtype, safe);
     }

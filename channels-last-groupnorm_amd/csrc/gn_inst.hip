@@ -78,6 +78,7 @@ template <typename K> int resident_slots(K kernel) {
 bool resident_tiling(const Plan &base, int64_t samples, int nv, int slots, Plan &out) {
   const int64_t columns = samples * base.nchunk;
   if (slots <= 0 || columns > slots || samples > 65535) return false;
+  if (base.G > 8192 || base.C >= (1 << 23)) return false;  // the kernels index their records with 24-bit multiplies
   const int64_t rows = (int64_t)nv * base.rpi;
   const int64_t tiles = (base.R + rows - 1) / rows;
   if (columns * tiles > slots) return false;
