@@ -8,6 +8,7 @@
 #include <time.h>
 
 #include <atomic>
+#include <mutex>
 #include <vector>
 
 #include "../../include/gnnhwc.h"
@@ -242,6 +243,63 @@ unsigned long long next_epoch() {
   unsigned long long e = seed + 0x9E3779B97F4A7C15ull * (counter.fetch_add(1) + 1);
   return e ? e : 1ull;
 }
+// ---- epochs of captured launches -------------------------------------------------------------------------
+// One generation word per device, in the library's own device memory (each device holds its own copy of the
+// array below at its own address; host code only ever uses the address hipGetSymbolAddress returns for the
+// current device, never the array's name).
+static __device__ __align__(256) unsigned long long g_generation_cell[32];
+__global__ void bump_generation_kernel(unsigned long long *generation) { *generation += 1; }
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_capture_mutex;
+unsigned long long *g_generation_ptr[kMaxDevices];
+bool g_generation_tried[kMaxDevices];
+unsigned long long g_last_capture[kMaxDevices];
+bool g_have_last_capture[kMaxDevices];
+std::atomic<unsigned long long> g_capture_sequence{0};
+}  // namespace
+unsigned long long CapturedEpoch::next_sequence() const { return g_capture_sequence.fetch_add(1) + 1; }
+bool captured_epoch(hipStream_t stream, CapturedEpoch &out) {
+  out.generation = nullptr;
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  unsigned long long id = 0;
+  if (hipStreamGetCaptureInfo(stream, &st, &id) != hipSuccess) {
+    (void)hipGetLastError();
+    return true;  // not a capturing stream as far as the runtime can tell
+  }
+  if (st == hipStreamCaptureStatusNone) return true;
+  if (st != hipStreamCaptureStatusActive) return false;  // invalidated capture: record nothing that depends on it
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();
+    return false;
+  }
+  std::lock_guard<std::mutex> lock(g_capture_mutex);
+  if (!g_generation_tried[dev]) {
+    g_generation_tried[dev] = true;
+    // looking a symbol up is not a stream operation, but keep the capture from seeing it as one
+    hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+    const bool swapped = hipThreadExchangeStreamCaptureMode(&mode) == hipSuccess;
+    void *p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_generation_cell)) != hipSuccess) {
+      (void)hipGetLastError();
+      p = nullptr;
+    }
+    if (swapped) (void)hipThreadExchangeStreamCaptureMode(&mode);
+    g_generation_ptr[dev] = (unsigned long long *)p;
+  }
+  unsigned long long *word = g_generation_ptr[dev];
+  if (!word) return false;
+  if (!g_have_last_capture[dev] || g_last_capture[dev] != id) {
+    hipLaunchKernelGGL(bump_generation_kernel, dim3(1), dim3(1), 0, stream, word);
+    if (hipGetLastError() != hipSuccess) return false;
+    g_have_last_capture[dev] = true;
+    g_last_capture[dev] = id;
+  }
+  out.generation = word;
+  return true;
+}
+
 bool trace_waits() {
   static const bool w = env_int("GNNHWC_TRACE", 0) != 2;
   return w;

@@ -60,14 +60,16 @@ __device__ __forceinline__ void trace_point(const SyncArea &s, int point, float 
 }
 
 // A launch recorded into a HIP graph is replayed with identical kernel arguments, so the host cannot give
-// each replay a fresh epoch.  For captured launches the host therefore records a one-thread kernel in front
-// that increments a generation word in the workspace header, and that counter is the epoch: it is different
-// for every captured launch that ever runs on this workspace, whatever graph it belongs to.  Bit 63 keeps the
-// two families apart: set for counter epochs, clear for the host's.
-template <int UNUSED> __global__ void bump_generation_kernel(unsigned long long *generation) { *generation += 1; }
+// each replay a fresh epoch.  The first captured launch of a capture therefore records a one-thread kernel in
+// front of itself that increments a generation word owned by the library (one per device), and the epoch of a
+// captured launch is that generation combined with a sequence number the host fixed at capture time (in
+// s.epoch): the generation differs between any two replays of any graphs, the sequence number between the
+// launches of one graph.  Bit 63 keeps the two families apart: set for captured launches, clear for the host's.
+constexpr int kCapturedSeqBits = 24;
 __device__ __forceinline__ SyncArea resident_epoch(SyncArea s) {
   constexpr unsigned long long kCaptured = 1ull << 63;
-  if (s.generation) s.epoch = kCaptured | *s.generation;
+  if (s.generation)
+    s.epoch = kCaptured | (*s.generation << kCapturedSeqBits) | (s.epoch & ((1ull << kCapturedSeqBits) - 1));
   else s.epoch &= ~kCaptured;
   if (s.epoch == 0) s.epoch = 1;
   return s;

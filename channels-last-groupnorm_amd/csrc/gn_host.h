@@ -64,9 +64,7 @@ inline BwdWorkspace bwd_workspace(const Plan &p) {
   w.total = w.compactG + align_up((size_t)p.N * p.G * 2, 64);
   return w;
 }
-// Every layout of the workspace (streaming or single-launch, forward or backward) leaves its first 256 bytes
-// alone: they hold the generation word of captured single-launch kernels, which must survive whatever else a
-// caller runs on the same workspace between two replays of a graph.
+// Every layout of the workspace (streaming or single-launch, forward or backward) leaves its first 256 bytes unused.
 constexpr size_t kWorkspaceHeader = 256;
 // The resident kernels keep their partial results and one flag per workgroup in the same workspace.
 constexpr int kMaxResidentBlocks = 4 * kNumCU;
@@ -88,6 +86,16 @@ inline size_t resident_bwd_bytes(int64_t chunk_channels, int64_t G) {
 }
 // A fresh nonzero 64-bit value per call (gn_api.hip).
 unsigned long long next_epoch();
+// Epoch source of launches that are being recorded into a HIP graph.  captured_epoch() leaves `generation` null
+// when `stream` is not capturing; otherwise it points at the library's per-device generation word, and the
+// kernel that increments it has been recorded on `stream` if this is the first such launch of the capture.
+// Returns false if the stream is capturing but the word is not available (the caller then records the
+// multi-launch kernels instead).
+struct CapturedEpoch {
+  const unsigned long long *generation = nullptr;
+  unsigned long long next_sequence() const;  // differs between the captured launches of one graph
+};
+bool captured_epoch(hipStream_t stream, CapturedEpoch &out);
 bool resident_enabled();
 // Device buffer for in-kernel timestamps when GNNHWC_TRACE=1, else null.
 unsigned long long *trace_buffer();

@@ -93,24 +93,11 @@ bool resident_tiling(const Plan &base, int64_t samples, int nv, int slots, Plan 
 
 struct ResidentWorkspace {
   SyncArea sync;
-  unsigned long long *generation;  // device word in the workspace header
 };
-// True while `stream` is recording into a HIP graph.
-bool stream_is_capturing(hipStream_t stream) {
-  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(stream, &st) != hipSuccess) {
-    (void)hipGetLastError();
-    return false;
-  }
-  return st != hipStreamCaptureStatusNone;
-}
-// Captured launches get their per-replay epoch from a generation word bumped by a kernel recorded in front.
-void arm_generation(ResidentWorkspace &r, hipStream_t stream) {
-  r.sync.generation = nullptr;
-  if (stream_is_capturing(stream)) {
-    hipLaunchKernelGGL(bump_generation_kernel<GN_INST_DTYPE>, dim3(1), dim3(1), 0, stream, r.generation);
-    r.sync.generation = r.generation;
-  }
+// Captured launches take their per-replay epoch from the library's generation word and a sequence number.
+void arm_generation(ResidentWorkspace &r, const CapturedEpoch &c) {
+  r.sync.generation = c.generation;
+  if (c.generation) r.sync.epoch = c.next_sequence();
 }
 ResidentWorkspace resident_fwd_ws(void *ws, const Plan &p) {
   ResidentWorkspace r;
@@ -120,7 +107,7 @@ ResidentWorkspace resident_fwd_ws(void *ws, const Plan &p) {
   r.sync.crecs = nullptr;
   r.sync.crec_bytes = 0;
   r.sync.status = resident_status();
-  r.generation = (unsigned long long *)ws;
+  r.sync.generation = nullptr;
   r.sync.max_spins = resident_spin_limit();
   r.sync.epoch = next_epoch();
   r.sync.trace = trace_buffer();
@@ -136,7 +123,7 @@ ResidentWorkspace resident_bwd_ws(void *ws, const Plan &p) {
   r.sync.recs = base + resident_crec_bytes(cc);
   r.sync.rec_bytes = (unsigned)resident_rec_bytes(p.G);
   r.sync.status = resident_status();
-  r.generation = (unsigned long long *)ws;
+  r.sync.generation = nullptr;
   r.sync.max_spins = resident_spin_limit();
   r.sync.epoch = next_epoch();
   r.sync.trace = trace_buffer();
@@ -167,13 +154,15 @@ template <typename PT, int ACT, int NV> bool try_resident_fwd_nv(const FwdArgs &
   Plan p;
   if (!resident_tiling(a.plan, per, NV, slots, p)) return false;
   if (!resident_status()) return false;
+  CapturedEpoch cap;
+  if (!captured_epoch(a.stream, cap)) return false;
   mark_resident_launch();
   const int64_t sample = a.plan.R * a.plan.C;
   for (int64_t n0 = 0; n0 < a.plan.N; n0 += per) {
     Plan pb = p;
     if (a.plan.N - n0 < per) resident_tiling(a.plan, a.plan.N - n0, NV, slots, pb);  // the last, shorter group
     ResidentWorkspace r = resident_fwd_ws(a.ws, pb);  // the launches follow each other on the stream: same records
-    arm_generation(r, a.stream);
+    arm_generation(r, cap);
     launch(kKindFusedFwd, kernel, tile_grid(pb, 0), dim3(kBlock), a.stream, (const elem_t *)a.x + n0 * sample,
            (elem_t *)a.y + n0 * sample, r.sync, a.w, a.b, a.mean ? (char *)a.mean + n0 * a.plan.G * stat_size(a.sdtype) : nullptr,
            a.rstd ? (char *)a.rstd + n0 * a.plan.G * stat_size(a.sdtype) : nullptr, a.sdtype, (A)a.eps, pb);
@@ -213,6 +202,8 @@ template <typename PT, int ACT, int NV> bool try_resident_bwd_nv(const BwdArgs &
   const size_t crec_need = (size_t)a.plan.N * p.tiles * a.plan.C * 16;
   if (crec_need > resident_crec_bytes((int64_t)p.lpr * p.vec)) return false;
   if (!resident_status()) return false;
+  CapturedEpoch cap;
+  if (!captured_epoch(a.stream, cap)) return false;
   mark_resident_launch();
   const int64_t sample = a.plan.R * a.plan.C;
   const size_t ssz = stat_size(a.sdtype);
@@ -221,7 +212,7 @@ template <typename PT, int ACT, int NV> bool try_resident_bwd_nv(const BwdArgs &
     if (a.plan.N - n0 < per) resident_tiling(a.plan, a.plan.N - n0, NV, slots, pb);  // the last, shorter group
     pb.tiles = p.tiles;  // same row tiling in every group (it depends on R and NV only)
     ResidentWorkspace r = resident_bwd_ws(a.ws, pb);
-    arm_generation(r, a.stream);
+    arm_generation(r, cap);
     const bool last = n0 + per >= a.plan.N;
     launch(kKindFusedBwd, kernel, tile_grid(pb, 0), dim3(kBlock), a.stream, (const elem_t *)a.x + n0 * sample,
            (const elem_t *)a.dy + n0 * sample, (elem_t *)a.dx + n0 * sample, (const char *)a.mean + n0 * a.plan.G * ssz,

@@ -482,3 +482,69 @@ def test_hip_graph_replay(family, shape, G, device):
             assert torch.equal(got, ref), "replay %d: %s differs from the eager result" % (rep, name)
         step()  # eager work on the same workspaces between replays
         torch.cuda.synchronize()
+
+
+@pytest.mark.gpu
+def test_hip_graphs_share_a_workspace(device):
+    """Captured single-launch kernels take their epoch from a per-replay generation and a per-launch sequence
+    number.  Two launches of the same shape on ONE workspace inside one graph (different inputs), and two graphs
+    that share that workspace and are replayed alternately with eager calls in between, must each reproduce the
+    eager results bit for bit: a launch that mistook another launch's records for its own would normalise with
+    the wrong statistics."""
+    gen = torch.Generator().manual_seed(33)
+    shape, G = (2, 320, 32, 32), 32
+    N, C = shape[0], shape[1]
+    xs = [nrc_view(channels_last_like(shape, torch.bfloat16, device, gen, 1.0 + i, 0.5 * i)) for i in range(3)]
+    dy = nrc_view(channels_last_like(shape, torch.bfloat16, device, gen))
+    w = (torch.rand(C, generator=gen) + 0.5).to(torch.bfloat16).to(device)
+    b = (0.1 * torch.randn(C, generator=gen)).to(torch.bfloat16).to(device)
+    lib = _cabi.lib
+    R = xs[0].shape[1]
+    nbytes = max(lib.gnnhwc_fwd_workspace_bytes(N, R, C, G, 3), lib.gnnhwc_bwd_workspace_bytes(N, R, C, G, 3))
+    ws = torch.empty((nbytes,), dtype=torch.uint8, device=device)
+    ys = [torch.empty_like(xs[0]) for _ in xs]
+    dx = torch.empty_like(xs[0])
+
+    def step_a():  # two forwards of the same shape on the same workspace, then a backward on it
+        _, m0, r0 = cabi_fwd(xs[0], w, b, G, 1e-5, 2, y=ys[0], ws=ws)
+        _, m1, r1 = cabi_fwd(xs[1], w, b, G, 1e-5, 2, y=ys[1], ws=ws)
+        _, dw, db = cabi_bwd(dy, xs[1], w, b, m1, r1, G, 2, dx=dx, ws=ws)
+        return m0, r0, m1, r1, dw, db
+
+    def step_b():
+        _, m2, r2 = cabi_fwd(xs[2], w, b, G, 1e-5, 2, y=ys[2], ws=ws)
+        return m2, r2
+
+    outs_a = step_a()
+    outs_b = step_b()
+    torch.cuda.synchronize()
+    want_a = [t.clone() for t in (ys[0], ys[1], dx) + tuple(outs_a)]
+    want_b = [t.clone() for t in (ys[2],) + tuple(outs_b)]
+    assert not torch.equal(want_a[0], want_a[1])
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step_a()
+        step_b()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    ga, gb = torch.cuda.CUDAGraph(), torch.cuda.CUDAGraph()
+    with torch.cuda.graph(ga):
+        got_a = step_a()
+    with torch.cuda.graph(gb):
+        got_b = step_b()
+    for rep in range(3):
+        for t in ys + [dx] + list(got_a) + list(got_b):
+            t.fill_(float("nan"))
+        ga.replay()
+        gb.replay()
+        if rep == 1:
+            ga.replay()  # the same graph twice in a row
+        torch.cuda.synchronize()
+        for i, (got, ref) in enumerate(zip((ys[0], ys[1], dx) + tuple(got_a), want_a)):
+            assert torch.equal(got, ref), "replay %d: output %d of the first graph differs from the eager result" % (rep, i)
+        for i, (got, ref) in enumerate(zip((ys[2],) + tuple(got_b), want_b)):
+            assert torch.equal(got, ref), "replay %d: output %d of the second graph differs from the eager result" % (rep, i)
+        step_b()  # eager work on the same workspace between replays
+        torch.cuda.synchronize()
+
