@@ -164,6 +164,44 @@ _op_lib.impl("fwd", _fwd_meta, "Meta")
 _op_lib.impl("bwd", _bwd_meta, "Meta")
 
 
+def _fwd_setup_context(ctx, inputs, output):
+    X, weight, bias, G, _eps, act_fn_option = inputs
+    _Y, means, rstds = output
+    ctx.save_for_backward(X, weight, bias, means, rstds)
+    ctx.G = G
+    ctx.act_fn_option = act_fn_option
+    ctx.mark_non_differentiable(means, rstds)
+
+
+def _fwd_backward(ctx, dY, _dmeans, _drstds):
+    X, weight, bias, means, rstds = ctx.saved_tensors
+    dY = dY.permute(0, 2, 1).contiguous().permute(0, 2, 1)  # X's own (R*C, 1, C) strides
+    dX, dweight, dbias = torch.ops.gnop.bwd(dY, X, weight, bias, means, rstds, ctx.G, ctx.act_fn_option)
+    return dX, dweight, dbias, None, None, None
+
+
+# Autograd formula of gnop::fwd itself (the reference only differentiates through GN_NHWC_Func, custom_gn.py:29-47):
+# with it and the meta kernels above, code that calls the operator directly can be traced and compiled whole.
+torch.library.register_autograd("gnop::fwd", _fwd_backward, setup_context=_fwd_setup_context, lib=_op_lib)
+
+
+def group_norm_nhwc(x, weight, bias, num_groups, eps=1e-5, activation="identity"):
+    """Functional, traceable form of GN_NHWC.forward for channels-last input (x.stride(1) == 1): the same operator
+    and results, differentiated through the operator's registered autograd formula instead of GN_NHWC_Func, so
+    torch.compile can keep it in one graph.  weight / bias must be given (use ones / zeros for a non-affine norm)."""
+    if x.stride(1) != 1:
+        raise RuntimeError("group_norm_nhwc expects channels-last input (stride 1 along dim 1)")
+    nd = x.dim()
+    x = x.permute(0, *range(2, nd), 1).contiguous()  # (N, *spatial, C), a no-op copy-wise for channels-last input
+    shape = x.shape
+    R = 1
+    for d in shape[1:-1]:
+        R *= d
+    X_flat = x.view(shape[0], R, shape[-1]).permute(0, 2, 1)
+    Y, _means, _rstds = torch.ops.gnop.fwd(X_flat, weight, bias, num_groups, eps, ACTIVATION_CODES[activation])
+    return Y.permute(0, 2, 1).reshape(shape).permute(0, nd - 1, *range(1, nd - 1))
+
+
 class GN_NHWC_Func(torch.autograd.Function):
     """custom_gn.py:29-47.  apply(X, weight, bias, G, eps, activation_code) -> Y with X's shape and strides."""
 

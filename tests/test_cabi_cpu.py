@@ -142,3 +142,23 @@ def test_operator_metadata_on_meta_tensors():
         assert mean.shape == (N, G) and rstd.shape == (N, G) and mean.dtype == sdtype
         dX, dw, db = torch.ops.gnop.bwd(X, X, w, w, mean, rstd, G, 2)
         assert dX.shape == (N, C, R) and dX.stride() == (R * C, 1, C) and dw.shape == (C,) and db.dtype == dtype
+
+
+def test_operator_autograd_on_meta_tensors():
+    """gnop::fwd carries its own autograd formula: differentiating through the traceable functional form on meta
+    tensors yields gradients of the right shapes, dtypes and strides without running a kernel."""
+    from gnnhwc import group_norm_nhwc
+
+    N, C, H, W, G = 2, 8, 5, 3, 4
+    x = torch.empty((N, H, W, C), dtype=torch.bfloat16, device="meta").permute(0, 3, 1, 2).requires_grad_()
+    w = torch.empty((C,), dtype=torch.bfloat16, device="meta", requires_grad=True)
+    b = torch.empty((C,), dtype=torch.bfloat16, device="meta", requires_grad=True)
+    y = group_norm_nhwc(x, w, b, G, 1e-5, "silu")
+    assert y.shape == x.shape and y.stride() == x.stride() and y.dtype == x.dtype
+    gx, gw, gb = torch.autograd.grad(y, (x, w, b), torch.empty_like(y))
+    assert gx.shape == x.shape and gx.stride() == x.stride()
+    assert gw.shape == (C,) and gb.shape == (C,) and gw.dtype == torch.bfloat16
+    with pytest.raises(RuntimeError):
+        group_norm_nhwc(torch.empty((N, C, H, W), device="meta"), w, b, G)
+    with pytest.raises(KeyError):
+        group_norm_nhwc(x, w, b, G, 1e-5, "tanh")

@@ -548,3 +548,36 @@ def test_hip_graphs_share_a_workspace(device):
         step_b()  # eager work on the same workspace between replays
         torch.cuda.synchronize()
 
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_functional_form_traces_into_one_graph(dtype, device):
+    """group_norm_nhwc under torch.compile (fullgraph, so any graph break fails; the 'aot_eager' backend traces
+    forward and backward with fake tensors and then runs the traced graphs, i.e. the HIP operators): outputs and
+    all three gradients equal the module's bit for bit (same kernels, same inputs)."""
+    from gnnhwc import group_norm_nhwc
+
+    gen = torch.Generator().manual_seed(5)
+    shape, G = (2, 64, 24, 24), 8
+    x0 = channels_last_like(shape, dtype, device, gen, 1.3, 0.2)
+    dy = channels_last_like(shape, dtype, device, gen)
+    m = GN_NHWC(G, shape[1], activation="silu").to(device=device, dtype=dtype)
+    with torch.no_grad():
+        m.weight.copy_((torch.rand(shape[1], generator=gen) + 0.5).to(dtype))
+        m.bias.copy_((0.1 * torch.randn(shape[1], generator=gen)).to(dtype))
+    x = x0.clone().requires_grad_()
+    y = m(x)
+    gx, gw, gb = torch.autograd.grad(y, (x, m.weight, m.bias), dy)
+
+    def fn(t, w, b):
+        return group_norm_nhwc(t * 1.0, w, b, G, m.eps, "silu")
+
+    compiled = torch.compile(fn, backend="aot_eager", fullgraph=True)
+    x2 = x0.clone().requires_grad_()
+    w2 = m.weight.detach().clone().requires_grad_()
+    b2 = m.bias.detach().clone().requires_grad_()
+    y2 = compiled(x2, w2, b2)
+    assert y2.stride() == y.stride()
+    gx2, gw2, gb2 = torch.autograd.grad(y2, (x2, w2, b2), dy)
+    assert torch.equal(y2, y) and torch.equal(gx2, gx) and torch.equal(gw2, gw) and torch.equal(gb2, gb)
