@@ -300,6 +300,46 @@ bool captured_epoch(hipStream_t stream, CapturedEpoch &out) {
   return true;
 }
 
+// ---- one single-launch kernel at a time per device ----------------------------------------------------------
+namespace {
+std::mutex g_order_mutex;
+hipStream_t g_order_stream[kMaxDevices];
+bool g_order_have[kMaxDevices];
+hipEvent_t g_order_event[kMaxDevices];
+}  // namespace
+ResidentOrder::ResidentOrder(hipStream_t stream, bool capturing) : locked_(false) {
+  if (capturing) return;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();
+    return;
+  }
+  g_order_mutex.lock();
+  locked_ = true;
+  if (g_order_have[dev] && g_order_stream[dev] != stream) {
+    hipEvent_t &ev = g_order_event[dev];
+    if (!ev && hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) {
+      (void)hipGetLastError();
+      ev = nullptr;
+    }
+    // the event covers everything submitted to the previous stream so far, the last single-launch kernel included;
+    // a previous stream that has started recording a graph since is left alone (an event recorded there would
+    // become part of that graph)
+    hipStreamCaptureStatus prev = hipStreamCaptureStatusNone;
+    const bool known = hipStreamIsCapturing(g_order_stream[dev], &prev) == hipSuccess;
+    if (ev && known && prev == hipStreamCaptureStatusNone && hipEventRecord(ev, g_order_stream[dev]) == hipSuccess) {
+      if (hipStreamWaitEvent(stream, ev, 0) != hipSuccess) (void)hipGetLastError();
+    } else {
+      (void)hipGetLastError();  // e.g. the previous stream no longer exists
+    }
+  }
+  g_order_stream[dev] = stream;
+  g_order_have[dev] = true;
+}
+ResidentOrder::~ResidentOrder() {
+  if (locked_) g_order_mutex.unlock();
+}
+
 bool trace_waits() {
   static const bool w = env_int("GNNHWC_TRACE", 0) != 2;
   return w;

@@ -96,6 +96,22 @@ struct CapturedEpoch {
   unsigned long long next_sequence() const;  // differs between the captured launches of one graph
 };
 bool captured_epoch(hipStream_t stream, CapturedEpoch &out);
+// Two single-launch kernels must not share the device: each needs all of its workgroups resident at once.  Kernels
+// of one stream follow each other anyway; when a call arrives on another stream than the previous single-launch
+// call of the device, this makes the new stream wait for everything submitted so far on the previous one (an
+// event recorded there, no host synchronisation).  The object also serialises the host-side bookkeeping and the
+// enqueueing of the launches it guards, so it lives until they have been submitted.  Launches that are being
+// recorded into a graph are not ordered this way.
+class ResidentOrder {
+ public:
+  ResidentOrder(hipStream_t stream, bool capturing);
+  ~ResidentOrder();
+  ResidentOrder(const ResidentOrder &) = delete;
+  ResidentOrder &operator=(const ResidentOrder &) = delete;
+
+ private:
+  bool locked_;
+};
 bool resident_enabled();
 // Device buffer for in-kernel timestamps when GNNHWC_TRACE=1, else null.
 unsigned long long *trace_buffer();

@@ -156,6 +156,7 @@ template <typename PT, int ACT, int NV> bool try_resident_fwd_nv(const FwdArgs &
   if (!resident_status()) return false;
   CapturedEpoch cap;
   if (!captured_epoch(a.stream, cap)) return false;
+  ResidentOrder order(a.stream, cap.generation != nullptr);
   mark_resident_launch();
   const int64_t sample = a.plan.R * a.plan.C;
   for (int64_t n0 = 0; n0 < a.plan.N; n0 += per) {
@@ -204,6 +205,7 @@ template <typename PT, int ACT, int NV> bool try_resident_bwd_nv(const BwdArgs &
   if (!resident_status()) return false;
   CapturedEpoch cap;
   if (!captured_epoch(a.stream, cap)) return false;
+  ResidentOrder order(a.stream, cap.generation != nullptr);
   mark_resident_launch();
   const int64_t sample = a.plan.R * a.plan.C;
   const size_t ssz = stat_size(a.sdtype);

@@ -110,9 +110,12 @@ int gnnhwc_bwd(const void *dy, const void *x, const void *weight, const void *bi
  * Kernel selection (no counterpart in the reference).  By default a problem whose tensors fit in the
  * register files of one launch is run by the single-launch kernels (x and dy are read from memory once;
  * workgroups exchange partial results while resident), anything else by the multi-launch streaming
- * kernels.  The single-launch kernels assume no second such launch is running on another stream of the
- * same device at the same time; gnnhwc_set_resident(0) (or GNNHWC_DISABLE_RESIDENT=1 in the environment)
- * forces the streaming kernels.  Process-wide; returns the previous setting.
+ * kernels.  A single-launch kernel needs the device to itself among its kind: calls of one process on
+ * different streams are ordered by the library (a call on another stream than the previous single-launch
+ * call of the device first makes its stream wait, on the device, for what has been submitted to that
+ * previous stream), but launches recorded into graphs that are replayed concurrently, and other processes
+ * on the same device, are not; gnnhwc_set_resident(0) (or GNNHWC_DISABLE_RESIDENT=1 in the environment)
+ * forces the streaming kernels, which have no such requirement.  Process-wide; returns the previous setting.
  */
 int gnnhwc_set_resident(int on);
 

@@ -581,3 +581,47 @@ def test_functional_form_traces_into_one_graph(dtype, device):
     assert y2.stride() == y.stride()
     gx2, gw2, gb2 = torch.autograd.grad(y2, (x2, w2, b2), dy)
     assert torch.equal(y2, y) and torch.equal(gx2, gx) and torch.equal(gw2, gw) and torch.equal(gb2, gb)
+
+
+@pytest.mark.gpu
+def test_two_streams_take_turns(device):
+    """Single-launch kernels issued on two streams with no host synchronisation in between: the library orders each
+    behind the previous one on the other stream (each needs the whole device to itself), so every call reproduces
+    the result of the same call made alone, and no call reports a failed wait."""
+    lib = _cabi.lib
+    gen = torch.Generator().manual_seed(44)
+    cases = []
+    for shape, G in (((1, 640, 64, 64), 32), ((2, 320, 64, 64), 32)):
+        C = shape[1]
+        x = nrc_view(channels_last_like(shape, torch.bfloat16, device, gen, 1.5, 0.3))
+        dy = nrc_view(channels_last_like(shape, torch.bfloat16, device, gen))
+        w = (torch.rand(C, generator=gen) + 0.5).to(torch.bfloat16).to(device)
+        b = (0.1 * torch.randn(C, generator=gen)).to(torch.bfloat16).to(device)
+        cases.append((x, dy, w, b, G))
+
+    def step(case):
+        x, dy, w, b, G = case
+        y, mean, rstd = cabi_fwd(x, w, b, G, 1e-5, 2)
+        dx, dw, db = cabi_bwd(dy, x, w, b, mean, rstd, G, 2)
+        return y, mean, rstd, dx, dw, db
+
+    before = _cabi.set_resident(True)
+    prev = lib.gnnhwc_debug_set_spin_limit(50000)  # a wait that cannot succeed ends within a fraction of a second
+    try:
+        want = [step(c) for c in cases]
+        torch.cuda.synchronize()
+        streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+        got = []
+        for it in range(40):
+            for s, c in zip(streams, cases):
+                with torch.cuda.stream(s):
+                    got.append(step(c))
+        torch.cuda.synchronize()
+        for i, out in enumerate(got):
+            for a, ref in zip(out, want[i % 2]):
+                assert torch.equal(a, ref), "call %d differs from the same call made alone" % i
+        step(cases[0])  # a failed wait would be reported by the next call
+        torch.cuda.synchronize()
+    finally:
+        lib.gnnhwc_debug_set_spin_limit(prev)
+        _cabi.set_resident(before)
