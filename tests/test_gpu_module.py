@@ -625,3 +625,59 @@ def test_two_streams_take_turns(device):
     finally:
         lib.gnnhwc_debug_set_spin_limit(prev)
         _cabi.set_resident(before)
+
+
+def _device_err(a, truth):
+    """err() of the harness, evaluated on the device (for tensors too large to bring to the host)."""
+    a = a.reshape(-1).double()
+    t = truth.reshape(-1).double()
+    rms = float(t.square().mean().sqrt()) or 1.0
+    return float(((a - t).abs() / (t.abs() + rms)).max())
+
+
+@pytest.mark.gpu
+def test_more_than_two_to_the_31_elements(device):
+    """(5, 2048 * 2048, 128) bf16 holds 2.7e9 elements: element offsets of the last two samples do not fit 32 bits
+    (the reference indexes with int, gn_kernel.cu:21, and overflows here).  Statistics are per sample, so each
+    checked sample must agree with the same sample run alone (a tensor whose offsets are small) and with float64
+    statistics computed by torch on the device; dgamma / dbeta must be the sum of the single-sample results, and
+    dx must sum to zero over every (sample, group) slab."""
+    N, R, C, G = 5, 2048 * 2048, 128, 32
+    D = C // G
+    assert N * R * C > 2 ** 31
+    gen = torch.Generator(device=device).manual_seed(7)
+    x = torch.empty((N, R, C), dtype=torch.bfloat16, device=device)
+    dy = torch.empty((N, R, C), dtype=torch.bfloat16, device=device)
+    for n in range(N):
+        x[n] = (torch.randn((R, C), generator=gen, device=device) * (1.0 + 0.5 * n) + 0.3 * n).to(torch.bfloat16)
+        dy[n] = torch.randn((R, C), generator=gen, device=device).to(torch.bfloat16)
+    w = (torch.rand(C, generator=gen, device=device) + 0.5).to(torch.bfloat16)
+    b = (0.1 * torch.randn(C, generator=gen, device=device)).to(torch.bfloat16)
+    y, mean, rstd = cabi_fwd(x, w, b, G, 1e-5, 2)
+    dx, dw, db = cabi_bwd(dy, x, w, b, mean, rstd, G, 2)
+    torch.cuda.synchronize()
+    dw_sum = torch.zeros(C, dtype=torch.float64, device=device)
+    db_sum = torch.zeros(C, dtype=torch.float64, device=device)
+    for n in range(N):
+        xs, dys = x[n:n + 1], dy[n:n + 1]
+        y1, m1, r1 = cabi_fwd(xs, w, b, G, 1e-5, 2)
+        # dgamma / dbeta of one sample in float32, so that their sum can be compared with the bf16 result
+        dx1, dw1, db1 = cabi_bwd(dys, xs, w.float(), b.float(), m1, r1, G, 2)
+        dw_sum += dw1.double()
+        db_sum += db1.double()
+        if n in (0, N - 2, N - 1):
+            xd = xs.double().view(R, G, D)
+            mu = xd.mean(dim=(0, 2))
+            var = xd.var(dim=(0, 2), correction=0)
+            del xd
+            assert _device_err(mean[n], mu) <= 1e-5 and _device_err(rstd[n], (var + 1e-5).rsqrt()) <= 1e-5
+            assert _device_err(mean[n], m1[0]) <= 1e-5 and _device_err(rstd[n], r1[0]) <= 1e-5
+            assert _device_err(y[n], y1[0]) <= 2.0 ** -7, "sample %d: y differs from the sample run alone" % n
+            assert _device_err(dx[n], dx1[0]) <= 2.0 ** -6, "sample %d: dx differs from the sample run alone" % n
+            slab = dx[n].double().view(R, G, D)
+            total = slab.sum(dim=(0, 2)).abs().max()
+            scale = slab.abs().sum(dim=(0, 2)).max()
+            del slab
+            # every element of dx carries a bf16 rounding error of relative size 2^-9 with random sign
+            assert float(total) <= float(scale) * 2.0 ** -9 * 8 / (R * D) ** 0.5
+    assert _device_err(dw, dw_sum) <= 2.0 ** -7 and _device_err(db, db_sum) <= 2.0 ** -7
