@@ -48,6 +48,9 @@ def parse_args():
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-shape warm / cold / copy-ceiling table")
     ap.add_argument("--graph", action="store_true", help="time the replay of a HIP graph of the K steps instead of eager launches")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
+    ap.add_argument("--fused-add", action="store_true",
+                    help="also time gnnhwc_fwd_add (residual + sum output fused into the forward) against an elementwise "
+                         "addition followed by gnnhwc_fwd, per shape (reported under 'fused_add')")
     ap.add_argument("--counter-workload", action="store_true",
                     help="no timing: one 256 MiB plain copy (calibration) and a few fwd+bwd calls per shape, for a rocprofv3 --pmc run")
     return ap.parse_args()
@@ -333,6 +336,67 @@ def cpu_baseline(cfg_names, seconds):
     }
 
 
+def fused_add_table(names, device, steps, warmup):
+    """Forward with the skip-connection addition fused in (reads x and the residual, writes their sum and y:
+    4 S algorithmic bytes) against the unfused sequence a caller of the plain forward runs (torch.add into a sum
+    buffer, then gnnhwc_fwd on it: 3 S + 2 S), and the channel-bias-only form (2 S) against its unfused sequence."""
+    import torch
+    from tests import configs
+
+    out = {}
+    for n in names:
+        cfg = configs.CONFIGS[n]
+        p = Problem(cfg, device)
+        b = p.sets[0]
+        x = b["x"]
+        res = (0.5 * torch.randn(x.shape, device=device)).to(x.dtype)
+        cb = torch.randn((p.N, p.C), device=device).to(x.dtype)
+        total = torch.empty_like(x)
+        stream_of = lambda: torch.cuda.current_stream().cuda_stream  # noqa: E731
+
+        def call_add(residual, channel_bias, sum_out):
+            rc = p.lib.gnnhwc_fwd_add(x.data_ptr(), residual.data_ptr() if residual is not None else None,
+                                      channel_bias.data_ptr() if channel_bias is not None else None,
+                                      sum_out.data_ptr() if sum_out is not None else None, p.w.data_ptr(), p.b.data_ptr(),
+                                      b["y"].data_ptr(), p.mean.data_ptr(), p.rstd.data_ptr(), p.N, p.R, p.C, p.G, 1e-5,
+                                      p.act, p.dt, p.dt, p.sdt, p.dt, p.ws_f.data_ptr(), p.ws_f.numel(), stream_of())
+            if rc != 0:
+                raise RuntimeError(p.lib.gnnhwc_last_error().decode())
+
+        def plain_on(t):
+            rc = p.lib.gnnhwc_fwd(t.data_ptr(), p.w.data_ptr(), p.b.data_ptr(), b["y"].data_ptr(), p.mean.data_ptr(),
+                                  p.rstd.data_ptr(), p.N, p.R, p.C, p.G, 1e-5, p.act, p.dt, p.dt, p.sdt,
+                                  p.ws_f.data_ptr(), p.ws_f.numel(), stream_of())
+            if rc != 0:
+                raise RuntimeError(p.lib.gnnhwc_last_error().decode())
+
+        def unfused_residual():
+            torch.add(x, res, out=total)
+            plain_on(total)
+
+        def unfused_bias():
+            torch.add(x, cb[:, None, :], out=total)
+            plain_on(total)
+
+        cases = {
+            "residual_sum_fused": (lambda: call_add(res, None, total), 4),
+            "residual_sum_unfused": (unfused_residual, 4),
+            "channel_bias_fused": (lambda: call_add(None, cb, None), 2),
+            "channel_bias_unfused": (unfused_bias, 2),
+        }
+        r = {}
+        for key, (fn, streams) in cases.items():
+            t = min(time_region(fn, steps, warmup, False) for _ in range(3)) / steps
+            r[key + "_us"] = round(t * 1e6, 3)
+            r[key + "_gbps"] = round(streams * p.S / t / 1e9, 1)  # algorithmic bytes of the FUSED form / time
+        r["residual_sum_speedup"] = round(r["residual_sum_unfused_us"] / r["residual_sum_fused_us"], 3)
+        r["channel_bias_speedup"] = round(r["channel_bias_unfused_us"] / r["channel_bias_fused_us"], 3)
+        out[n] = r
+        del p
+        torch.cuda.empty_cache()
+    return out
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -455,6 +519,8 @@ def main():
         "roofline": roofline,
         "shapes": shapes,
     }
+    if args.fused_add:
+        line["fused_add"] = fused_add_table(head_names, device, max(20, args.steps // 2), args.warmup)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(head_names, args.cpu_seconds)
     print(json.dumps(line))

@@ -438,9 +438,9 @@ size_t gnnhwc_bwd_workspace_bytes(int64_t N, int64_t R, int64_t C, int64_t G, in
   return align_up(bwd_ws_bytes(N, R, C, G, dtype), 256);
 }
 
-int gnnhwc_fwd(const void *x, const void *weight, const void *bias, void *y, void *mean, void *rstd, int64_t N,
-               int64_t R, int64_t C, int64_t G, double eps, int act, int dtype, int param_dtype, int stats_dtype,
-               void *workspace, size_t workspace_bytes, void *stream) {
+static int forward(const void *x, const AddArgs &add, const void *weight, const void *bias, void *y, void *mean, void *rstd,
+                   int64_t N, int64_t R, int64_t C, int64_t G, double eps, int act, int dtype, int param_dtype,
+                   int stats_dtype, void *workspace, size_t workspace_bytes, void *stream) {
   int rc = check_shape(N, R, C, G, dtype);
   if (rc != GNNHWC_OK) return rc;
   rc = check_dtypes(dtype, param_dtype, stats_dtype);
@@ -456,8 +456,9 @@ int gnnhwc_fwd(const void *x, const void *weight, const void *bias, void *y, voi
     return fail(GNNHWC_ERR_WORKSPACE, "forward workspace must be 16-byte aligned and at least %zu bytes (got %p, %zu bytes)",
                 need, workspace, workspace_bytes);
   const int vec = 16 / elem_size(dtype);
-  const bool vector_ok = C % vec == 0 && aligned16(x) && aligned16(y);
+  const bool vector_ok = C % vec == 0 && aligned16(x) && aligned16(y) && aligned16(add.residual) && aligned16(add.sum_out);
   FwdArgs a;
+  a.add = add;
   a.x = x; a.w = weight; a.b = bias; a.y = y; a.mean = mean; a.rstd = rstd;
   a.eps = eps; a.act = act; a.pdtype = param_dtype; a.sdtype = stats_dtype;
   a.ws = workspace; a.stream = (hipStream_t)stream;
@@ -472,6 +473,27 @@ int gnnhwc_fwd(const void *x, const void *weight, const void *bias, void *y, voi
   }
   if (e != hipSuccess) return fail(GNNHWC_ERR_LAUNCH, "forward launch failed: %s", hipGetErrorString(e));
   return GNNHWC_OK;
+}
+
+int gnnhwc_fwd(const void *x, const void *weight, const void *bias, void *y, void *mean, void *rstd, int64_t N,
+               int64_t R, int64_t C, int64_t G, double eps, int act, int dtype, int param_dtype, int stats_dtype,
+               void *workspace, size_t workspace_bytes, void *stream) {
+  const AddArgs none = {nullptr, nullptr, GN_F32, nullptr};
+  return forward(x, none, weight, bias, y, mean, rstd, N, R, C, G, eps, act, dtype, param_dtype, stats_dtype, workspace,
+                 workspace_bytes, stream);
+}
+
+int gnnhwc_fwd_add(const void *x, const void *residual, const void *channel_bias, void *sum_out, const void *weight,
+                   const void *bias, void *y, void *mean, void *rstd, int64_t N, int64_t R, int64_t C, int64_t G,
+                   double eps, int act, int dtype, int param_dtype, int stats_dtype, int channel_bias_dtype,
+                   void *workspace, size_t workspace_bytes, void *stream) {
+  if (channel_bias && channel_bias_dtype != dtype && !(channel_bias_dtype == GN_F32 && (dtype == GN_F16 || dtype == GN_BF16)))
+    return fail(GNNHWC_ERR_INVALID_ARGUMENT, "channel_bias_dtype must equal dtype, or be F32 for F16/BF16 data");
+  if (sum_out && sum_out == y)
+    return fail(GNNHWC_ERR_INVALID_ARGUMENT, "sum_out and y must be different buffers");
+  const AddArgs add = {residual, channel_bias, channel_bias ? channel_bias_dtype : GN_F32, sum_out};
+  return forward(x, add, weight, bias, y, mean, rstd, N, R, C, G, eps, act, dtype, param_dtype, stats_dtype, workspace,
+                 workspace_bytes, stream);
 }
 
 int gnnhwc_bwd(const void *dy, const void *x, const void *weight, const void *bias, const void *mean, const void *rstd,
@@ -582,7 +604,8 @@ int gnnhwc_debug_copy(void *dst, const void *src, size_t bytes, void *stream) {
 
 const char *gnnhwc_kernel_kind_name(int kind) {
   static const char *names[GNNHWC_NUM_KERNEL_KINDS] = {"fwd_stats", "fwd_stats_compact", "fwd_apply", "bwd_reduce",
-                                                       "bwd_compact", "bwd_dx", "fused_fwd", "fused_bwd", "copy"};
+                                                       "bwd_compact", "bwd_dx", "fused_fwd", "fused_bwd", "copy",
+                                                       "fwd_add", "fused_fwd_add"};
   return (kind >= 0 && kind < GNNHWC_NUM_KERNEL_KINDS) ? names[kind] : "";
 }
 

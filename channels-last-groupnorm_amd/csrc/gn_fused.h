@@ -171,10 +171,17 @@ __device__ __forceinline__ void for_group_records(const SyncArea &s, __amdgpu_bu
 // the per-lane moments are an exact two-pass computation.
 //   records : {mean, M2, epoch} per (n, chunk, group, tile)
 // ---------------------------------------------------------------------------------------------
-template <typename T, typename PT, int VEC, int ACT, int NV>
-__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 8 ? 4 : NV <= 16 ? 3 : 2))) void fused_fwd_kernel(
+// ADD: 0 plain forward; 1 a per-(sample, channel) addend only (same register budget as the plain kernel);
+// 2 a residual tensor, with or without the addend (holds two tiles while it combines them, like the backward).
+constexpr int kAddNone = 0, kAddChannel = 1, kAddResidual = 2;
+// Occupancy the register budget is sized for.
+constexpr int fused_fwd_waves(int nv, int add) {
+  return add == kAddResidual ? (nv <= 4 ? 4 : nv <= 8 ? 3 : nv <= 16 ? 2 : 1) : (nv <= 8 ? 4 : nv <= 16 ? 3 : 2);
+}
+template <typename T, typename PT, int VEC, int ACT, int NV, int ADD>
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fwd_waves(NV, ADD)))) void fused_fwd_kernel(
     const T *__restrict__ x, T *__restrict__ y, SyncArea sync_arg, const void *w, const void *b, void *mean_out,
-    void *rstd_out, int sdtype, acc_t<T> eps, Plan p) {
+    void *rstd_out, int sdtype, acc_t<T> eps, AddArgs add, Plan p) {
   using A = acc_t<T>;
   using LV = LaneVec<T, VEC>;
   const SyncArea sync = resident_epoch(sync_arg);
@@ -196,12 +203,61 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 8 
     const int cvi = l.cvi < p.cv ? l.cvi : p.cv - 1;
     lane_params_flat<A, PT, VEC>(cvi * VEC, w, b, sync.recs, sa, sb);
   }
+  // ADD: the per-(sample, channel) addend of the lane's channels, requested with the parameters and without branches
+  A tb[VEC];
+  if constexpr (ADD != kAddNone) {
+    const int cvi = l.cvi < p.cv ? l.cvi : p.cv - 1;
+    const void *cb = add.channel_bias ? add.channel_bias : sync.recs;
+    const int64_t cb0 = add.channel_bias ? n * p.C + (int64_t)cvi * VEC : 0;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const A v = load_scalar_flat<A>(cb, add.channel_bias ? cb0 + j : 0, add.channel_bias_dtype, sync.recs);
+      tb[j] = add.channel_bias ? v : (A)0;
+    }
+  }
   issue_order_fence();
   if (rows > 0) {
     // every load is unconditional (rows past the lane's last one re-read it): the waits that follow can then
     // count loads exactly, and row u is processed while rows u + 1 ... are still in flight
+    if constexpr (ADD == kAddResidual) {
+      // (an absent residual would re-read x and be discarded, so that the loads stay free of branches; the host
+      // picks the channel-only variant for that case)
+      const T *rp = add.residual ? (const T *)add.residual : x;
+      const bool has_r = add.residual != nullptr;
+      typename LV::raw_t rbuf[NV];
 #pragma unroll
-    for (int u = 0; u < NV; ++u) buf[u] = LV::load(x + off + (int64_t)clamp_row(u, rows) * step);
+      for (int u = 0; u < NV; ++u) {
+        const int64_t o = off + (int64_t)clamp_row(u, rows) * step;
+        buf[u] = LV::load(x + o);
+        rbuf[u] = LV::load(rp + o);
+      }
+      T *so = (T *)add.sum_out;
+#pragma unroll
+      for (int u = 0; u < NV; ++u) {
+        A vx[VEC], vr[VEC];
+        LV::unpack(buf[u], vx);
+        LV::unpack(rbuf[u], vr);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) vx[j] = (vx[j] + (has_r ? vr[j] : (A)0)) + tb[j];
+        buf[u] = LV::pack(vx);  // rounded to T once: the statistics and y are those of the stored sum
+        if (so && u < rows) LV::store(so + off + (int64_t)u * step, buf[u]);
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < NV; ++u) buf[u] = LV::load(x + off + (int64_t)clamp_row(u, rows) * step);
+      if constexpr (ADD == kAddChannel) {
+        T *so = (T *)add.sum_out;
+#pragma unroll
+        for (int u = 0; u < NV; ++u) {
+          A vx[VEC];
+          LV::unpack(buf[u], vx);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) vx[j] += tb[j];
+          buf[u] = LV::pack(vx);
+          if (so && u < rows) LV::store(so + off + (int64_t)u * step, buf[u]);
+        }
+      }
+    }
   }
   // everything up to the exchange is on the critical path of the whole group; what follows it is not: a wavefront
   // still working towards the exchange goes before one (of another workgroup on the same SIMD) that is past it

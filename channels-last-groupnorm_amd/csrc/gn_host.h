@@ -19,11 +19,15 @@ enum KernelKind {
   kKindFusedFwd = 6,
   kKindFusedBwd = 7,
   kKindCopy = 8,
+  kKindAdd = 9,        // elementwise pre-addition of the multi-launch fused-addition forward
+  kKindFusedFwdAdd = 10,  // single-launch forward with the pre-addition fused in
   kNumKinds = 9
 };
 
 struct FwdArgs {
   const void *x, *w, *b;
+  AddArgs add;  // all null: plain forward
+  bool has_add() const { return add.residual || add.channel_bias || add.sum_out; }
   void *y, *mean, *rstd;
   double eps;
   int act, pdtype, sdtype;

@@ -7,6 +7,14 @@
 #ifndef GN_INST_DTYPE
 #error "compile with -DGN_INST_DTYPE=<0|1|2|3>"
 #endif
+// One data type's kernels are spread over three translation units so that they compile in parallel:
+// part 0 the forward, part 1 the backward, part 2 the forward with fused additions (single-launch variants).
+#ifndef GN_INST_PART
+#error "compile with -DGN_INST_PART=<0|1|2>"
+#endif
+#define GN_PART_FWD (GN_INST_PART == 0)
+#define GN_PART_BWD (GN_INST_PART == 1)
+#define GN_PART_ADD (GN_INST_PART == 2)
 
 namespace gn {
 
@@ -40,6 +48,7 @@ dim3 tile_grid(const Plan &p, int extra_x) {
   return dim3((unsigned)(p.tiles + extra_x), (unsigned)p.nchunk, (unsigned)(p.N < 65535 ? p.N : 65535));
 }
 
+#if GN_PART_FWD
 template <typename PT, int VEC, int ACT> void launch_apply(const FwdArgs &a, const A *part, const PartialGeo &q) {
   const Plan &p = a.plan;
   launch(kKindFwdApply, (apply_kernel<elem_t, PT, VEC, ACT>), tile_grid(p, 0), dim3(kBlock), a.stream, (const elem_t *)a.x,
@@ -54,6 +63,7 @@ template <typename PT, int VEC> void launch_apply_act(const FwdArgs &a, const A 
     default: launch_apply<PT, VEC, GN_ACT_GELU_TANH>(a, part, q); break;
   }
 }
+#endif  // GN_PART_FWD
 
 // ---- resident (single-launch) path ----------------------------------------------------------------
 // Workgroups that can be resident at once for a kernel: occupancy reported by the runtime times the CUs.
@@ -145,10 +155,11 @@ int worthwhile_batches(const Plan &p, bool backward) {
 }
 size_t stat_size(int sdtype) { return sdtype == GN_F32 ? 4 : sdtype == GN_F64 ? 8 : 2; }
 
+#if !GN_PART_BWD
 // One NV variant, the tensor cut into `batches` launches over consecutive samples (1: the whole tensor).
-template <typename PT, int ACT, int NV> bool try_resident_fwd_nv(const FwdArgs &a, int batches) {
+template <typename PT, int ACT, int NV, int ADD> bool try_resident_fwd_nv(const FwdArgs &a, int batches) {
   if (NV < resident_min_rows()) return false;
-  auto kernel = fused_fwd_kernel<elem_t, PT, kVec, ACT, NV>;
+  auto kernel = fused_fwd_kernel<elem_t, PT, kVec, ACT, NV, ADD>;
   static const int slots = resident_slots(kernel);
   const int64_t per = (a.plan.N + batches - 1) / batches;
   Plan p;
@@ -164,19 +175,35 @@ template <typename PT, int ACT, int NV> bool try_resident_fwd_nv(const FwdArgs &
     if (a.plan.N - n0 < per) resident_tiling(a.plan, a.plan.N - n0, NV, slots, pb);  // the last, shorter group
     ResidentWorkspace r = resident_fwd_ws(a.ws, pb);  // the launches follow each other on the stream: same records
     arm_generation(r, cap);
-    launch(kKindFusedFwd, kernel, tile_grid(pb, 0), dim3(kBlock), a.stream, (const elem_t *)a.x + n0 * sample,
-           (elem_t *)a.y + n0 * sample, r.sync, a.w, a.b, a.mean ? (char *)a.mean + n0 * a.plan.G * stat_size(a.sdtype) : nullptr,
-           a.rstd ? (char *)a.rstd + n0 * a.plan.G * stat_size(a.sdtype) : nullptr, a.sdtype, (A)a.eps, pb);
+    AddArgs add = a.add;  // this group of samples' part of the addends
+    if (add.residual) add.residual = (const elem_t *)add.residual + n0 * sample;
+    if (add.sum_out) add.sum_out = (elem_t *)add.sum_out + n0 * sample;
+    if (add.channel_bias) add.channel_bias = (const char *)add.channel_bias + n0 * a.plan.C * stat_size(add.channel_bias_dtype);
+    launch(ADD != kAddNone ? kKindFusedFwdAdd : kKindFusedFwd, kernel, tile_grid(pb, 0), dim3(kBlock), a.stream,
+           (const elem_t *)a.x + n0 * sample, (elem_t *)a.y + n0 * sample, r.sync, a.w, a.b,
+           a.mean ? (char *)a.mean + n0 * a.plan.G * stat_size(a.sdtype) : nullptr,
+           a.rstd ? (char *)a.rstd + n0 * a.plan.G * stat_size(a.sdtype) : nullptr, a.sdtype, (A)a.eps, add, pb);
   }
   return true;
 }
-template <typename PT, int ACT> bool try_resident_fwd_act(const FwdArgs &a) {
-  const int most = a.plan.N < worthwhile_batches(a.plan, false) ? (int)a.plan.N : worthwhile_batches(a.plan, false);
+template <typename PT, int ACT, int ADD> bool try_resident_fwd_add(const FwdArgs &a) {
+  // with a residual the launch holds two tensors, as the backward does, and the alternative is three launches:
+  // the backward's rule for cutting the batch into several single-launch kernels applies
+  const int wb = worthwhile_batches(a.plan, ADD == kAddResidual);
+  const int most = a.plan.N < wb ? (int)a.plan.N : wb;
   for (int b = 1; b <= most; ++b)
-    if (try_resident_fwd_nv<PT, ACT, 4>(a, b) || try_resident_fwd_nv<PT, ACT, 8>(a, b) ||
-        try_resident_fwd_nv<PT, ACT, 16>(a, b) || try_resident_fwd_nv<PT, ACT, 32>(a, b))
+    if (try_resident_fwd_nv<PT, ACT, 4, ADD>(a, b) || try_resident_fwd_nv<PT, ACT, 8, ADD>(a, b) ||
+        try_resident_fwd_nv<PT, ACT, 16, ADD>(a, b) || try_resident_fwd_nv<PT, ACT, 32, ADD>(a, b))
       return true;
   return false;
+}
+template <typename PT, int ACT> bool try_resident_fwd_act(const FwdArgs &a) {
+#if GN_PART_ADD
+  // a sum of x and a channel addend alone, or a copy of x (sum_out only), needs no second tile
+  return a.add.residual ? try_resident_fwd_add<PT, ACT, kAddResidual>(a) : try_resident_fwd_add<PT, ACT, kAddChannel>(a);
+#else
+  return try_resident_fwd_add<PT, ACT, kAddNone>(a);
+#endif
 }
 template <typename PT> bool try_resident_fwd_pt(const FwdArgs &a) {
   switch (a.act) {
@@ -187,11 +214,25 @@ template <typename PT> bool try_resident_fwd_pt(const FwdArgs &a) {
     default: return try_resident_fwd_act<PT, GN_ACT_GELU_TANH>(a);
   }
 }
+}  // namespace
+// the single-launch forward with fused additions lives in part 2
+bool GN_CAT(try_resident_fwd_added_, GN_SUFFIX)(const FwdArgs &a);
+namespace {
 bool try_resident_fwd(const FwdArgs &a) {
-  if (!resident_enabled() || a.plan.vec == 1 || sizeof(A) != 4) return false;
-  return a.pdtype == GN_INST_DTYPE ? try_resident_fwd_pt<elem_t>(a) : try_resident_fwd_pt<wide_param_t>(a);
+  if constexpr (sizeof(A) != 4) {
+    return false;  // no single-launch kernels for 64-bit data
+  } else {
+    if (!resident_enabled() || a.plan.vec == 1) return false;
+#if GN_PART_FWD
+    if (a.has_add()) return GN_CAT(try_resident_fwd_added_, GN_SUFFIX)(a);
+#endif
+    return a.pdtype == GN_INST_DTYPE ? try_resident_fwd_pt<elem_t>(a) : try_resident_fwd_pt<wide_param_t>(a);
+  }
 }
 
+#endif  // !GN_PART_BWD
+
+#if GN_PART_BWD
 template <typename PT, int ACT, int NV> bool try_resident_bwd_nv(const BwdArgs &a, int batches) {
   if (NV < resident_min_rows()) return false;
   auto kernel = fused_bwd_kernel<elem_t, PT, kVec, ACT, NV>;
@@ -241,12 +282,31 @@ template <typename PT> bool try_resident_bwd_pt(const BwdArgs &a) {
   }
 }
 bool try_resident_bwd(const BwdArgs &a) {
-  if (!resident_enabled() || a.plan.vec == 1 || sizeof(A) != 4) return false;
-  return a.pdtype == GN_INST_DTYPE ? try_resident_bwd_pt<elem_t>(a) : try_resident_bwd_pt<wide_param_t>(a);
+  if constexpr (sizeof(A) != 4) {
+    return false;
+  } else {
+    if (!resident_enabled() || a.plan.vec == 1) return false;
+    return a.pdtype == GN_INST_DTYPE ? try_resident_bwd_pt<elem_t>(a) : try_resident_bwd_pt<wide_param_t>(a);
+  }
 }
 
+#endif  // GN_PART_BWD
+
+#if GN_PART_FWD
 template <int VEC> hipError_t fwd_impl(const FwdArgs &a) {
   if (VEC != 1 && try_resident_fwd(a)) return hipGetLastError();
+  if (a.has_add()) {
+    // multi-launch form: materialise the sum (in sum_out, or in y when the caller does not want it), then
+    // normalise it from there (in place when it sits in y)
+    const Plan &p = a.plan;
+    elem_t *dst = (elem_t *)(a.add.sum_out ? a.add.sum_out : a.y);
+    launch(kKindAdd, (add_kernel<elem_t, VEC>), tile_grid(p, 0), dim3(kBlock), a.stream, (const elem_t *)a.x, a.add, dst,
+           (const void *)a.ws, p);
+    FwdArgs plain = a;
+    plain.x = dst;
+    plain.add = AddArgs{nullptr, nullptr, a.add.channel_bias_dtype, nullptr};
+    return fwd_impl<VEC>(plain);
+  }
   const Plan &p = a.plan;
   const FwdWorkspace ws = fwd_workspace(p);
   A *base = (A *)((char *)a.ws + kWorkspaceHeader);
@@ -270,6 +330,9 @@ template <int VEC> hipError_t fwd_impl(const FwdArgs &a) {
   return hipGetLastError();
 }
 
+#endif  // GN_PART_FWD
+
+#if GN_PART_BWD
 template <typename PT, int VEC, int ACT> void launch_bwd_act(const BwdArgs &a) {
   const Plan &p = a.plan;
   const BwdWorkspace ws = bwd_workspace(p);
@@ -314,13 +377,20 @@ template <int VEC> hipError_t bwd_impl(const BwdArgs &a) {
   return hipGetLastError();
 }
 
+#endif  // GN_PART_BWD
+
 }  // namespace
 
+#if GN_PART_FWD
 hipError_t GN_CAT(launch_fwd_, GN_SUFFIX)(const FwdArgs &a) {
   return a.plan.vec == 1 ? fwd_impl<1>(a) : fwd_impl<kVec>(a);
 }
+#elif GN_PART_BWD
 hipError_t GN_CAT(launch_bwd_, GN_SUFFIX)(const BwdArgs &a) {
   return a.plan.vec == 1 ? bwd_impl<1>(a) : bwd_impl<kVec>(a);
 }
+#else
+bool GN_CAT(try_resident_fwd_added_, GN_SUFFIX)(const FwdArgs &a) { return try_resident_fwd(a); }
+#endif
 
 }  // namespace gn

@@ -411,6 +411,50 @@ __device__ __forceinline__ void block_channel_sums(const Plan &p, const LanePos 
 }
 
 // ---------------------------------------------------------------------------------------------
+// Pre-addition of the multi-launch forward: dst = x + residual + channel_bias[n][c], rounded to T once, on the
+// tiles of the streaming kernels.  dst may be x or the residual (a lane reads the elements it writes first, and no
+// other lane touches them).  `safe` is any readable 64 bytes (the workspace).
+// ---------------------------------------------------------------------------------------------
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlock) void add_kernel(const T *__restrict__ x, AddArgs add, T *dst, const void *safe, Plan p) {
+  using A = acc_t<T>;
+  using LV = LaneVec<T, VEC>;
+  constexpr int U = 4;  // rows of a lane in flight
+  const T *rp = (const T *)add.residual;
+  for (int64_t n = blockIdx.z; n < p.N; n += gridDim.z) {
+    const LanePos l = lane_pos(p, n, false);
+    if (l.rows == 0) continue;
+    A tb[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+      tb[j] = add.channel_bias ? load_scalar_flat<A>(add.channel_bias, n * p.C + (int64_t)l.cvi * VEC + j, add.channel_bias_dtype, safe)
+                               : (A)0;
+    const int64_t base = (n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC;
+    const int64_t step = (int64_t)p.rpi * p.C;
+    for (int r0 = 0; r0 < l.rows; r0 += U) {
+      typename LV::raw_t bx[U], br[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t o = base + (int64_t)clamp_row(r0 + u, l.rows) * step;
+        bx[u] = LV::load(x + o);
+        br[u] = LV::load((rp ? rp : x) + o);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (r0 + u < l.rows) {
+          A vx[VEC], vr[VEC];
+          LV::unpack(bx[u], vx);
+          LV::unpack(br[u], vr);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) vx[j] = (vx[j] + (rp ? vr[j] : (A)0)) + tb[j];
+          LV::store(dst + base + (int64_t)(r0 + u) * step, LV::pack(vx));
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 // Forward pass 1: per-tile (count, mean, M2) of every group the tile touches.
 // Does the work of compute_stats_pt1 (src/gnnhwc/csrc/gn_kernel.cu:132-224).
 //   part : 3 planes [N][nchunk][G][tiles]; only the groups a chunk intersects are written.

@@ -66,6 +66,16 @@ inline void set_divisors(Plan &p) {
   p.by_chunk = make_divisor((int64_t)p.lpr * p.vec, p.C + p.D);
 }
 
+// Pre-additions of the forward (fused-addition variant): the tensor that is normalised is s = x + residual + channel_bias[n][c],
+// rounded to T once (what an unfused elementwise addition in T would hand to the normalisation); s is written to
+// sum_out if that is given.  Any of the three pointers may be null.
+struct AddArgs {
+  const void *residual;      // (N, R, C) in T
+  const void *channel_bias;  // (N, C) in channel_bias_dtype
+  int channel_bias_dtype;
+  void *sum_out;             // (N, R, C) in T
+};
+
 // Geometry of a buffer of per-tile partial results as the consumer sees it: either the producer's own
 // (tiles, nchunk), or (1, 1) after the compaction kernel has merged all tiles of a sample.
 struct PartialGeo {

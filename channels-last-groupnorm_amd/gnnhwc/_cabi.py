@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(_CSRC, "libgnnhwc_hip.so")
 
 # dtype / activation codes of include/gnnhwc.h
 F32, F64, F16, BF16 = 0, 1, 2, 3
-NUM_KERNEL_KINDS = 9
+NUM_KERNEL_KINDS = 11
 
 SYMBOLS = (
     "gnnhwc_version",
@@ -20,6 +20,7 @@ SYMBOLS = (
     "gnnhwc_fwd_workspace_bytes",
     "gnnhwc_bwd_workspace_bytes",
     "gnnhwc_fwd",
+    "gnnhwc_fwd_add",
     "gnnhwc_bwd",
     "gnnhwc_profile_enable",
     "gnnhwc_profile_collect",
@@ -48,6 +49,8 @@ def _load():
     lib.gnnhwc_bwd_workspace_bytes.restype = sz
     lib.gnnhwc_fwd.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, dbl, ci, ci, ci, ci, vp, sz, vp]
     lib.gnnhwc_fwd.restype = ci
+    lib.gnnhwc_fwd_add.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, dbl, ci, ci, ci, ci, ci, vp, sz, vp]
+    lib.gnnhwc_fwd_add.restype = ci
     lib.gnnhwc_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, ci, ci, ci, ci, vp, sz, vp]
     lib.gnnhwc_bwd.restype = ci
     lib.gnnhwc_profile_enable.argtypes = [ci]

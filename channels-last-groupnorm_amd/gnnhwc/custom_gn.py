@@ -132,6 +132,59 @@ def gn_nhwc_bwd(dy, X, weight, bias, means, rstds, G, act_fn_option):
     return dX.permute(0, 2, 1), dweight, dbias
 
 
+def gn_nhwc_fwd_add(X, residual, channel_bias, weight, bias, G, eps, act_fn_option, return_sum):
+    """gnop::fwd_add (no counterpart in the reference): gnop::fwd of S = X + residual + channel_bias[:, :, None],
+    with the additions done inside the kernel.  X, residual: (N, C, R) channels-last views; channel_bias: (N, C).
+    Returns (Y, S, means, rstds); S has no elements unless return_sum."""
+    _check_device(X, "X")
+    _check_device(weight, "weight")
+    _check_device(bias, "bias")
+    if X.dim() != 3:
+        raise RuntimeError("gnop::fwd_add expects X of shape (N, C, R), got %s" % (tuple(X.shape),))
+    N, C, R = X.shape
+    dt = _dtype_code(X, "X")
+    pdt = _dtype_code(weight, "weight")
+    if bias.dtype != weight.dtype:
+        raise RuntimeError("weight and bias must have the same dtype (%s vs %s)" % (weight.dtype, bias.dtype))
+    if weight.numel() != C or bias.numel() != C:
+        raise RuntimeError("weight and bias must have %d elements" % C)
+    X_nrc = _as_nrc(X)
+    res_ptr = cb_ptr = None
+    cb_dt = dt
+    if residual is not None:
+        _check_device(residual, "residual")
+        if residual.shape != X.shape or residual.dtype != X.dtype:
+            raise RuntimeError("residual must have X's shape and dtype")
+        res_nrc = _as_nrc(residual)
+        res_ptr = res_nrc.data_ptr()
+    if channel_bias is not None:
+        _check_device(channel_bias, "channel_bias")
+        if tuple(channel_bias.shape) != (N, C):
+            raise RuntimeError("channel_bias must have shape (N, C) = (%d, %d)" % (N, C))
+        cb_dt = _dtype_code(channel_bias, "channel_bias")
+        channel_bias = channel_bias.contiguous()
+        cb_ptr = channel_bias.data_ptr()
+    Y = torch.empty_like(X_nrc)
+    S = torch.empty_like(X_nrc) if return_sum else torch.empty((N, 0, C), dtype=X.dtype, device=X.device)
+    sdtype = _stats_dtype(X.dtype)
+    means = torch.empty((N, G), dtype=sdtype, device=X.device)
+    rstds = torch.empty((N, G), dtype=sdtype, device=X.device)
+    lib = _cabi.lib
+    with torch.cuda.device(X.device):
+        nbytes = lib.gnnhwc_fwd_workspace_bytes(N, R, C, G, dt)
+        if nbytes == 0:
+            raise RuntimeError("gnop::fwd_add: " + _cabi.last_error())
+        ws = _workspace(nbytes, X.device)
+        rc = lib.gnnhwc_fwd_add(
+            X_nrc.data_ptr(), res_ptr, cb_ptr, S.data_ptr() if return_sum else None,
+            weight.contiguous().data_ptr(), bias.contiguous().data_ptr(),
+            Y.data_ptr(), means.data_ptr(), rstds.data_ptr(),
+            N, R, C, G, float(eps), int(act_fn_option), dt, pdt, _DTYPE_CODE[sdtype], cb_dt,
+            ws.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream)
+    _cabi.check(rc, "gnop::fwd_add")
+    return Y.permute(0, 2, 1), S.permute(0, 2, 1), means, rstds
+
+
 # TORCH_LIBRARY(gnop, m) { m.def("fwd", ...); m.def("bwd", ...); } -- custom_gn.cpp:91-94.  The reference
 # registers catch-all kernels that themselves reject non-device tensors; CompositeExplicitAutograd plays that
 # role here, so a CPU tensor reaches the "must be a CUDA tensor" check instead of a dispatcher error.
@@ -139,7 +192,10 @@ _op_lib = torch.library.Library("gnop", "DEF")
 _op_lib.define("fwd(Tensor X, Tensor weight, Tensor bias, int G, float eps, int act_fn_option) -> (Tensor, Tensor, Tensor)")
 _op_lib.define("bwd(Tensor dy, Tensor X, Tensor weight, Tensor bias, Tensor means, Tensor rstds, int G, "
                "int act_fn_option) -> (Tensor, Tensor, Tensor)")
+_op_lib.define("fwd_add(Tensor X, Tensor? residual, Tensor? channel_bias, Tensor weight, Tensor bias, int G, float eps, "
+               "int act_fn_option, bool return_sum) -> (Tensor, Tensor, Tensor, Tensor)")
 _op_lib.impl("fwd", gn_nhwc_fwd, "CompositeExplicitAutograd")
+_op_lib.impl("fwd_add", gn_nhwc_fwd_add, "CompositeExplicitAutograd")
 _op_lib.impl("bwd", gn_nhwc_bwd, "CompositeExplicitAutograd")
 
 
@@ -158,10 +214,18 @@ def _bwd_meta(dy, X, weight, bias, means, rstds, G, act_fn_option):
     return dX, torch.empty((C,), dtype=weight.dtype, device=X.device), torch.empty((C,), dtype=weight.dtype, device=X.device)
 
 
+def _fwd_add_meta(X, residual, channel_bias, weight, bias, G, eps, act_fn_option, return_sum):
+    N, C, R = X.shape
+    Y, means, rstds = _fwd_meta(X, weight, bias, G, eps, act_fn_option)
+    S = torch.empty((N, R if return_sum else 0, C), dtype=X.dtype, device=X.device).permute(0, 2, 1)
+    return Y, S, means, rstds
+
+
 # The reference's operators cannot be traced (its forward is wrapped in torch._dynamo.disable, custom_gn.py:63);
 # with these the operators at least carry correct output metadata under fake-tensor tracing.
 _op_lib.impl("fwd", _fwd_meta, "Meta")
 _op_lib.impl("bwd", _bwd_meta, "Meta")
+_op_lib.impl("fwd_add", _fwd_add_meta, "Meta")
 
 
 def _fwd_setup_context(ctx, inputs, output):
@@ -185,10 +249,53 @@ def _fwd_backward(ctx, dY, _dmeans, _drstds):
 torch.library.register_autograd("gnop::fwd", _fwd_backward, setup_context=_fwd_setup_context, lib=_op_lib)
 
 
-def group_norm_nhwc(x, weight, bias, num_groups, eps=1e-5, activation="identity"):
+def _fwd_add_setup_context(ctx, inputs, output):
+    X, residual, channel_bias, weight, bias, G, _eps, act_fn_option, return_sum = inputs
+    _Y, S, means, rstds = output
+    # the backward differentiates the normalisation at S: kept if it was materialised, else rebuilt from the inputs
+    ctx.save_for_backward(S if return_sum else X, residual, channel_bias, weight, bias, means, rstds)
+    ctx.have_sum = return_sum
+    ctx.G = G
+    ctx.act_fn_option = act_fn_option
+    ctx.mark_non_differentiable(means, rstds)
+
+
+def _fwd_add_backward(ctx, dY, dS, _dmeans, _drstds):
+    first, residual, channel_bias, weight, bias, means, rstds = ctx.saved_tensors
+    if ctx.have_sum:
+        S = first
+    else:
+        acc = first.float() if first.dtype in (torch.float16, torch.bfloat16) else first
+        if residual is not None:
+            acc = acc + residual
+        if channel_bias is not None:
+            acc = acc + channel_bias.unsqueeze(-1)
+        S = acc.to(first.dtype)
+    S = S.permute(0, 2, 1).contiguous().permute(0, 2, 1)
+    dY = dY.permute(0, 2, 1).contiguous().permute(0, 2, 1)
+    dSum, dweight, dbias = torch.ops.gnop.bwd(dY, S, weight, bias, means, rstds, ctx.G, ctx.act_fn_option)
+    if ctx.have_sum and dS is not None:
+        dSum = dSum + dS
+    dres = dSum if residual is not None else None
+    dcb = None
+    if channel_bias is not None:
+        dcb = dSum.sum(dim=2, dtype=torch.float32).to(channel_bias.dtype)
+    return dSum, dres, dcb, dweight, dbias, None, None, None, None
+
+
+torch.library.register_autograd("gnop::fwd_add", _fwd_add_backward, setup_context=_fwd_add_setup_context, lib=_op_lib)
+
+
+def group_norm_nhwc(x, weight, bias, num_groups, eps=1e-5, activation="identity", residual=None, channel_bias=None,
+                    return_sum=False):
     """Functional, traceable form of GN_NHWC.forward for channels-last input (x.stride(1) == 1): the same operator
     and results, differentiated through the operator's registered autograd formula instead of GN_NHWC_Func, so
-    torch.compile can keep it in one graph.  weight / bias must be given (use ones / zeros for a non-affine norm)."""
+    torch.compile can keep it in one graph.  weight / bias must be given (use ones / zeros for a non-affine norm).
+
+    Optional fused additions (no counterpart in the reference): the normalised tensor becomes
+    s = x + residual + channel_bias[:, :, None, ...] (residual: x's shape; channel_bias: (N, C), e.g. a time
+    embedding), computed inside the kernel and rounded to x's dtype once; with return_sum=True the call returns
+    (y, s) so that s can serve as the next skip connection."""
     if x.stride(1) != 1:
         raise RuntimeError("group_norm_nhwc expects channels-last input (stride 1 along dim 1)")
     nd = x.dim()
@@ -198,8 +305,21 @@ def group_norm_nhwc(x, weight, bias, num_groups, eps=1e-5, activation="identity"
     for d in shape[1:-1]:
         R *= d
     X_flat = x.view(shape[0], R, shape[-1]).permute(0, 2, 1)
-    Y, _means, _rstds = torch.ops.gnop.fwd(X_flat, weight, bias, num_groups, eps, ACTIVATION_CODES[activation])
-    return Y.permute(0, 2, 1).reshape(shape).permute(0, nd - 1, *range(1, nd - 1))
+    code = ACTIVATION_CODES[activation]
+
+    def unflat(t):
+        return t.permute(0, 2, 1).reshape(shape).permute(0, nd - 1, *range(1, nd - 1))
+
+    if residual is None and channel_bias is None and not return_sum:
+        Y, _means, _rstds = torch.ops.gnop.fwd(X_flat, weight, bias, num_groups, eps, code)
+        return unflat(Y)
+    R_flat = None
+    if residual is not None:
+        if residual.shape != torch.Size([shape[0], shape[-1], *shape[1:-1]]):
+            raise RuntimeError("residual must have x's shape")
+        R_flat = residual.permute(0, *range(2, nd), 1).contiguous().view(shape[0], R, shape[-1]).permute(0, 2, 1)
+    Y, S, _means, _rstds = torch.ops.gnop.fwd_add(X_flat, R_flat, channel_bias, weight, bias, num_groups, eps, code, return_sum)
+    return (unflat(Y), unflat(S)) if return_sum else unflat(Y)
 
 
 class GN_NHWC_Func(torch.autograd.Function):

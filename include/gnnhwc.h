@@ -94,6 +94,29 @@ int gnnhwc_fwd(const void *x, const void *weight, const void *bias,
                void *workspace, size_t workspace_bytes, void *stream /* hipStream_t */);
 
 /*
+ * Forward with the additions that precede the normalisation fused in (no counterpart in the reference, whose
+ * callers add in a separate pass: in a diffusion ResNet block `h + temb[:, :, None, None]` before the second
+ * norm, and `shortcut + h` before the next block's first norm).  The tensor that is normalised is
+ *   s = x + residual + channel_bias[n][c]          (fp32 arithmetic, rounded to dtype once)
+ * i.e. exactly what an elementwise addition in dtype would have handed to gnnhwc_fwd; y, mean and rstd are those
+ * of gnnhwc_fwd applied to s.
+ *   residual      : (N, R, C) in dtype, or NULL.
+ *   channel_bias  : (N, C) in channel_bias_dtype (dtype, or GNNHWC_F32 for F16/BF16 data), or NULL.
+ *   sum_out       : (N, R, C) in dtype; receives s.  May be NULL when the caller does not need the sum, and may be
+ *                   the same buffer as x or residual (in-place accumulation); must differ from y.
+ * With all three NULL this is gnnhwc_fwd.  Workspace: gnnhwc_fwd_workspace_bytes.  y may alias x or residual.
+ * A later backward takes s as its x (gnnhwc_bwd knows nothing of the additions: the gradient of s is the gradient
+ * of x and of residual, and its sum over R is the gradient of channel_bias).
+ */
+int gnnhwc_fwd_add(const void *x, const void *residual, const void *channel_bias, void *sum_out,
+                   const void *weight, const void *bias,
+                   void *y, void *mean, void *rstd,
+                   int64_t N, int64_t R, int64_t C, int64_t G,
+                   double eps, int act,
+                   int dtype, int param_dtype, int stats_dtype, int channel_bias_dtype,
+                   void *workspace, size_t workspace_bytes, void *stream /* hipStream_t */);
+
+/*
  * Backward: given dy and the forward's inputs and statistics, recomputes the activation gradient and
  * returns dx (N,R,C), dweight (C) and dbias (C).
  * Replaces run_gn_bwd_kernels<T> (gn_kernel.h:26-41; gn_kernel.cu:932-1055).
@@ -127,9 +150,10 @@ int gnnhwc_set_resident(int on);
  * reports, for each kernel kind, the number of launches and the summed duration in milliseconds since
  * the last collect, then clears the record.  Kinds: 0 fwd statistics, 1 fwd statistics compaction
  * (many row tiles only), 2 fwd apply, 3 bwd reduce, 4 bwd compaction (many row tiles only), 5 bwd dx,
- * 6 single-launch fwd, 7 single-launch bwd, 8 the plain copy of gnnhwc_debug_copy.
+ * 6 single-launch fwd, 7 single-launch bwd, 8 the plain copy of gnnhwc_debug_copy, 9 the elementwise pre-addition
+ * of gnnhwc_fwd_add's multi-launch form, 10 single-launch fwd with the pre-addition fused in.
  */
-#define GNNHWC_NUM_KERNEL_KINDS 9
+#define GNNHWC_NUM_KERNEL_KINDS 11
 int gnnhwc_profile_enable(int on);
 int gnnhwc_profile_collect(int64_t *launches /* [GNNHWC_NUM_KERNEL_KINDS] */,
                            double *total_ms /* [GNNHWC_NUM_KERNEL_KINDS] */);

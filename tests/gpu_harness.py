@@ -41,6 +41,29 @@ def cabi_fwd(x_nrc, w, b, G, eps, act, stats_dtype=None, y=None, ws=None):
     return y, mean, rstd
 
 
+def cabi_fwd_add(x_nrc, residual, channel_bias, w, b, G, eps, act, want_sum=True, sum_out=None, y=None):
+    """gnnhwc_fwd_add on (N, R, C) device tensors.  Returns y, sum (or None), mean, rstd."""
+    N, R, C = x_nrc.shape
+    dt = DT_CODE[x_nrc.dtype]
+    sdtype = torch.float32 if x_nrc.dtype in (torch.float16, torch.bfloat16) else x_nrc.dtype
+    pdt = DT_CODE[w.dtype] if w is not None else dt
+    cbdt = DT_CODE[channel_bias.dtype] if channel_bias is not None else dt
+    y = torch.empty_like(x_nrc) if y is None else y
+    if sum_out is None and want_sum:
+        sum_out = torch.empty_like(x_nrc)
+    mean = torch.empty((N, G), dtype=sdtype, device=x_nrc.device)
+    rstd = torch.empty((N, G), dtype=sdtype, device=x_nrc.device)
+    lib = _cabi.lib
+    nbytes = lib.gnnhwc_fwd_workspace_bytes(N, R, C, G, dt)
+    assert nbytes > 0, _cabi.last_error()
+    ws = torch.empty((nbytes,), dtype=torch.uint8, device=x_nrc.device)
+    rc = lib.gnnhwc_fwd_add(_ptr(x_nrc), _ptr(residual), _ptr(channel_bias), _ptr(sum_out), _ptr(w), _ptr(b), _ptr(y),
+                            _ptr(mean), _ptr(rstd), N, R, C, G, float(eps), int(act), dt, pdt, DT_CODE[sdtype], cbdt,
+                            _ptr(ws), ws.numel(), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    _cabi.check(rc, "gnnhwc_fwd_add")
+    return y, sum_out, mean, rstd
+
+
 def cabi_bwd(dy_nrc, x_nrc, w, b, mean, rstd, G, act, dx=None, ws=None, want_dw=True, want_db=True):
     N, R, C = x_nrc.shape
     dt = DT_CODE[x_nrc.dtype]

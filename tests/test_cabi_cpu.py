@@ -22,7 +22,7 @@ def _declared_functions():
 
 def test_library_exports_every_declared_symbol():
     names = _declared_functions()
-    assert {"gnnhwc_fwd", "gnnhwc_bwd", "gnnhwc_fwd_workspace_bytes", "gnnhwc_bwd_workspace_bytes", "gnnhwc_last_error",
+    assert {"gnnhwc_fwd", "gnnhwc_fwd_add", "gnnhwc_bwd", "gnnhwc_fwd_workspace_bytes", "gnnhwc_bwd_workspace_bytes", "gnnhwc_last_error",
             "gnnhwc_version", "gnnhwc_profile_enable", "gnnhwc_profile_collect", "gnnhwc_kernel_kind_name",
             "gnnhwc_debug_read_trace", "gnnhwc_set_resident", "gnnhwc_debug_copy", "gnnhwc_debug_set_spin_limit"} <= set(names)
     lib = ctypes.CDLL(_cabi.LIB_PATH)
@@ -162,3 +162,27 @@ def test_operator_autograd_on_meta_tensors():
         group_norm_nhwc(torch.empty((N, C, H, W), device="meta"), w, b, G)
     with pytest.raises(KeyError):
         group_norm_nhwc(x, w, b, G, 1e-5, "tanh")
+
+
+def test_fused_addition_operator_on_meta_tensors():
+    """gnop::fwd_add (additions fused into the forward): output metadata and the shapes of all five gradients,
+    on meta tensors (no kernel runs)."""
+    from gnnhwc import group_norm_nhwc
+
+    N, C, H, W, G = 2, 8, 5, 3, 4
+    mk = lambda *shape: torch.empty(shape, dtype=torch.bfloat16, device="meta")  # noqa: E731
+    x = mk(N, H, W, C).permute(0, 3, 1, 2).requires_grad_()
+    r = mk(N, H, W, C).permute(0, 3, 1, 2).requires_grad_()
+    t = mk(N, C).requires_grad_()
+    w = mk(C).requires_grad_()
+    b = mk(C).requires_grad_()
+    y, s = group_norm_nhwc(x, w, b, G, 1e-5, "silu", residual=r, channel_bias=t, return_sum=True)
+    assert y.shape == x.shape and y.stride() == x.stride() and s.shape == x.shape and s.stride() == x.stride()
+    grads = torch.autograd.grad((y, s), (x, r, t, w, b), (torch.empty_like(y), torch.empty_like(s)))
+    assert [tuple(g.shape) for g in grads] == [tuple(x.shape), tuple(x.shape), (N, C), (C,), (C,)]
+    y2 = group_norm_nhwc(x, w, b, G, 1e-5, "silu", channel_bias=t)
+    gx, gt = torch.autograd.grad(y2, (x, t), torch.empty_like(y2))
+    assert gx.shape == x.shape and gt.shape == (N, C) and gt.dtype == torch.bfloat16
+    with pytest.raises(RuntimeError):
+        group_norm_nhwc(x, w, b, G, 1e-5, "silu", residual=mk(N, C, H, W + 1))
+
