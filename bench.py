@@ -437,6 +437,8 @@ def main():
     ms_per_step = t / args.steps * 1e3
     value = alg / (t / args.steps) / 1e9
     t_other = time_region(step, args.steps, args.warmup, not use_graph, reps=1)
+    # the same K steps five more times (no further warm-up): spread of the headline figure
+    repeats = [time_region(step, args.steps, 0, use_graph, reps=1) for _ in range(5)]
 
     # ---- per-kernel durations (HIP events on the launch stream) ----
     prof = kernel_profile(probs, max(20, args.steps // 4))
@@ -516,6 +518,8 @@ def main():
         # (benchmark.py:101,107); the same time expressed in that accounting, for comparison with its CSVs
         "reference_accounting_gbps": round(sum((8 if p.bwd else 3) * p.S for p in probs) / (t / args.steps) / 1e9, 1),
         ("eager_ms_per_step" if use_graph else "graph_replay_ms_per_step"): round(t_other / args.steps * 1e3, 5),
+        "repeat_ms_per_step": [round(r / args.steps * 1e3, 5) for r in repeats],
+        "repeat_median_gbps": round(alg / (statistics.median(repeats) / args.steps) / 1e9, 1),
         "roofline": roofline,
         "shapes": shapes,
     }
