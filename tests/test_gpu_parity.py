@@ -91,3 +91,60 @@ def test_config_parity(family, name, device):
     slab = as_np64(dx).reshape(N, R, cfg.G, C // cfg.G)
     ulp = {torch.float32: 2.0 ** -24, torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}[dtype]
     assert np.max(np.abs(slab.sum(axis=(1, 3))) / np.abs(slab).sum(axis=(1, 3))) < 4 * ulp
+
+
+def _medium_shapes(count, seed):
+    """Seeded sample of medium-sized problems (1 - 60 MB tensors) with awkward geometry: channels per group that do
+    not divide the 64-channel chunks, rows that do not fill the last tile, several samples, one group, G == C / 8."""
+    rng = np.random.RandomState(seed)
+    out = []
+    while len(out) < count:
+        D = int(rng.choice([1, 2, 3, 5, 8, 10, 12, 20, 40, 45, 64, 96, 160]))
+        G = int(rng.choice([1, 2, 4, 8, 16, 32, 64]))
+        C = D * G
+        if C % 8 != 0 or C > 2560:
+            continue
+        N = int(rng.randint(1, 7))
+        R = int(rng.choice([rng.randint(200, 20000), 64 * 64, 128 * 128, 96 * 96, 37 * 53]))
+        if not (5e5 <= N * R * C <= 3e7):
+            continue
+        out.append((N, R, C, G, ["identity", "relu", "silu", "gelu", "gelu_tanh"][len(out) % 5],
+                    [torch.bfloat16, torch.float32, torch.float16][len(out) % 3]))
+    return out
+
+
+@pytest.mark.parametrize("N,R,C,G,act,dtype", _medium_shapes(36, 31))
+def test_random_medium_shapes(family, N, R, C, G, act, dtype, device):
+    """The single-launch kernels' tilings (and the streaming ones) on shapes no configuration names.  Truth is
+    torch's own GroupNorm + activation + autograd in float64 on the device (the results contract; the C oracle would
+    need minutes for these sizes); bars as for the configurations."""
+    print("medium", family, N, R, C, G, act, dtype, flush=True)
+    gen = torch.Generator().manual_seed(N * 1000003 + R * 101 + C)
+    x = (torch.randn((N, R, C), generator=gen) * 1.7 + torch.randn((C,), generator=gen)).to(dtype).to(device)
+    dy = torch.randn((N, R, C), generator=gen).to(dtype).to(device)
+    w = (torch.rand((C,), generator=gen) + 0.5).to(dtype).to(device)
+    b = (0.1 * torch.randn((C,), generator=gen)).to(dtype).to(device)
+    code = orc.ACT_CODES[act]
+
+    def torch_ref(t):
+        xs = x.to(t).permute(0, 2, 1).contiguous().requires_grad_()
+        ws, bs = w.to(t).requires_grad_(), b.to(t).requires_grad_()
+        ys = orc.torch_act(act)(torch.nn.functional.group_norm(xs, G, ws, bs, EPS))
+        gx, gw, gb = torch.autograd.grad(ys, (xs, ws, bs), dy.to(t).permute(0, 2, 1))
+        return {"y": ys.detach().permute(0, 2, 1), "dx": gx.permute(0, 2, 1), "dw": gw, "db": gb}
+
+    truth = torch_ref(torch.float64)
+    own = torch_ref(dtype) if dtype != torch.float32 else None
+    y, mean, rstd = cabi_fwd(x, w, b, G, EPS, code)
+    dx, dw, db = cabi_bwd(dy, x, w, b, mean, rstd, G, code)
+    torch.cuda.synchronize()
+    xd = x.double().view(N, R, G, C // G)
+    assert err(mean, xd.mean(dim=(1, 3))) <= FP32_TOL
+    assert err(rstd, (xd.var(dim=(1, 3), correction=0) + EPS).rsqrt()) <= FP32_TOL
+    mask = None
+    if act == "relu":
+        a = (rstd.double().repeat_interleave(C // G, dim=1) * w.double()[None, :])
+        z = x.double() * a[:, None, :] + (b.double()[None, :] - mean.double().repeat_interleave(C // G, dim=1) * a)[:, None, :]
+        mask = (z.abs() > RELU_BAND).cpu().numpy()
+    for name, ours in (("y", y), ("dx", dx), ("dw", dw), ("db", db)):
+        _check(name, ours, as_np64(truth[name]), own and as_np64(own[name]), dtype, mask if name == "dx" else None)
