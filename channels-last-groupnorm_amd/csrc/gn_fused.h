@@ -240,7 +240,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
 #pragma unroll
         for (int j = 0; j < VEC; ++j) vx[j] = (vx[j] + (has_r ? vr[j] : (A)0)) + tb[j];
         buf[u] = LV::pack(vx);  // rounded to T once: the statistics and y are those of the stored sum
-        if (so && u < rows) LV::store(so + off + (int64_t)u * step, buf[u]);
+        if (so && u < rows) store_streaming<LV>(so + off + (int64_t)u * step, buf[u]);
       }
     } else {
 #pragma unroll
@@ -254,7 +254,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
 #pragma unroll
           for (int j = 0; j < VEC; ++j) vx[j] += tb[j];
           buf[u] = LV::pack(vx);
-          if (so && u < rows) LV::store(so + off + (int64_t)u * step, buf[u]);
+          if (so && u < rows) store_streaming<LV>(so + off + (int64_t)u * step, buf[u]);
         }
       }
     }
@@ -352,7 +352,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
         LV::unpack(buf[u], v);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) v[j] = act_fwd<ACT, A>(v[j] * sa[j] + sb[j]);
-        LV::store(y + off + (int64_t)u * step, LV::pack(v));
+        store_streaming<LV>(y + off + (int64_t)u * step, LV::pack(v));
       }
     }
   }
@@ -577,7 +577,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
         LV::unpack(bd[u], vd);  // g'
 #pragma unroll
         for (int j = 0; j < VEC; ++j) vd[j] = sa[j] * vd[j] + (c1[j] * vx[j] + c2[j]);
-        LV::store(dx + off + (int64_t)u * step, LV::pack(vd));
+        store_streaming<LV>(dx + off + (int64_t)u * step, LV::pack(vd));
       }
     }
   }

@@ -719,7 +719,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
         else LV::unpack(buf1[u], v);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) v[j] = act_fwd<ACT, A>(v[j] * sa[j] + sb[j]);
-        if (bi * U + u < rows) LV::store(y + off + (int64_t)(bi * U + u) * step, LV::pack(v));
+        if (bi * U + u < rows) store_streaming<LV>(y + off + (int64_t)(bi * U + u) * step, LV::pack(v));
       }
     };
     // order of issue: the few small loads the prologue depends on first, then the first batch of x, so that
@@ -1052,7 +1052,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
           const A g = vd[j] * act_bwd<ACT, A>(vx[j] * sa[j] + sb[j]);
           vd[j] = sa[j] * g + (c1[j] * vx[j] + c2[j]);
         }
-        if (bi * U + u < rows) LV::store(dx + off + (int64_t)(bi * U + u) * step, LV::pack(vd));
+        if (bi * U + u < rows) store_streaming<LV>(dx + off + (int64_t)(bi * U + u) * step, LV::pack(vd));
       }
     };
     EarlyPartials<A, 2> early;
