@@ -428,6 +428,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
 #pragma unroll
         for (int u = 0; u < NV; ++u) {
           A vx[VEC], vd[VEC];
+          pin(bx[u]);  // one row at a time: cheap activations otherwise tempt the scheduler into unpacking many
+          pin(bd[u]);  // rows ahead, which costs more registers than the tile itself
           LV::unpack(bx[u], vx);
           LV::unpack(bd[u], vd);
 #pragma unroll
@@ -444,6 +446,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
         for (int u = 0; u < NV; ++u) {
           const A keep = u < rows ? (A)1 : (A)0;
           A vx[VEC], vd[VEC];
+          pin(bx[u]);
+          pin(bd[u]);
           LV::unpack(bx[u], vx);
           LV::unpack(bd[u], vd);
 #pragma unroll
