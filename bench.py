@@ -190,30 +190,39 @@ def measure_shape(prob_warm, prob_cold, steps, warmup, use_graph):
 
 
 def kernel_profile(probs, steps):
-    """{shape: {kind: mean us}}: `steps` back-to-back eager steps per shape with a HIP event pair bound to every
-    launch on the launch stream (begin-to-end time of each dispatch), collected once per shape."""
+    """{shape: {kind: (mean us per launch, launches per call)}} with a HIP event pair bound to every launch of one
+    shape at a time on the launch stream (begin-to-end time of each dispatch), while the whole workload runs in the
+    order of the timed region: every kernel is measured in the cache state and queue position it has there."""
     import torch
     from gnnhwc import _cabi
 
     stream = torch.cuda.current_stream().cuda_stream
     out = {}
     torch.cuda.synchronize()
-    _cabi.profile_enable(True)
+
+    def sweeps(target, count):
+        for _ in range(count):
+            for p in probs:
+                if p is target:
+                    _cabi.profile_enable(True)
+                    p.step(0, stream)
+                    _cabi.profile_enable(False)
+                else:
+                    p.step(0, stream)
+
     try:
-        for p in probs:
-            for _ in range(steps):  # untimed pass: creates the event pool, so that the host keeps ahead of the GPU below
-                p.step(0, stream)
+        for target in probs:
+            sweeps(target, steps)  # untimed pass: creates the event pool, so that the host keeps ahead of the GPU below
             _cabi.profile_collect()
             best = {}
             for _ in range(3):  # three passes, the fastest mean of each kind: robust against a transient slow start
-                for _ in range(steps):
-                    p.step(0, stream)
+                sweeps(target, steps)
                 res = _cabi.profile_collect()
                 for k, (n, ms) in res.items():
                     if n and (k not in best or ms / n < best[k][0] / best[k][1]):
                         best[k] = (ms, n)
             # mean per launch, and launches per call (a call may run one kernel kind several times, over groups of samples)
-            out[p.cfg.name] = {k: (ms / n * 1e3, n / steps) for k, (ms, n) in best.items()}
+            out[target.cfg.name] = {k: (ms / n * 1e3, n / steps) for k, (ms, n) in best.items()}
     finally:
         _cabi.profile_enable(False)
     return out
