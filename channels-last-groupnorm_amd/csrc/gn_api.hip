@@ -602,6 +602,22 @@ int gnnhwc_debug_copy(void *dst, const void *src, size_t bytes, void *stream) {
   return GNNHWC_OK;
 }
 
+int gnnhwc_debug_plan(int64_t N, int64_t R, int64_t C, int64_t G, int dtype, int vector, int backward, int64_t *out) {
+  if (!out) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "null output array");
+  const int rc = check_shape(N, R, C, G, dtype);
+  if (rc != GNNHWC_OK) return rc;
+  if (N == 0 || R == 0) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "empty problem: nothing is planned");
+  const int vec = 16 / elem_size(dtype);
+  if (vector && C % vec != 0) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "C = %lld is not a multiple of the vector width %d", (long long)C, vec);
+  const Plan p = make_plan(N, R, C, G, vector ? vec : 1, backward ? 2 : 1);
+  const size_t elems = backward ? bwd_workspace(p).total : fwd_workspace(p).total;
+  out[0] = p.vec; out[1] = p.cv; out[2] = p.lpr; out[3] = p.nchunk; out[4] = p.rpi; out[5] = p.tile_rows;
+  out[6] = p.tiles; out[7] = p.gmax; out[8] = p.nblocks; out[9] = needs_compaction(p) ? 1 : 0;
+  out[10] = (int64_t)(kWorkspaceHeader + elems * acc_size(dtype));
+  out[11] = p.D;
+  return GNNHWC_OK;
+}
+
 const char *gnnhwc_kernel_kind_name(int kind) {
   static const char *names[GNNHWC_NUM_KERNEL_KINDS] = {"fwd_stats", "fwd_stats_compact", "fwd_apply", "bwd_reduce",
                                                        "bwd_compact", "bwd_dx", "fused_fwd", "fused_bwd", "copy",

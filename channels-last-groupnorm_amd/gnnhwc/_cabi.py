@@ -27,6 +27,7 @@ SYMBOLS = (
     "gnnhwc_kernel_kind_name",
     "gnnhwc_set_resident",
     "gnnhwc_debug_read_trace",
+    "gnnhwc_debug_plan",
 )
 
 
@@ -65,6 +66,8 @@ def _load():
     lib.gnnhwc_debug_set_spin_limit.restype = ci
     lib.gnnhwc_debug_copy.argtypes = [vp, vp, sz, vp]
     lib.gnnhwc_debug_copy.restype = ci
+    lib.gnnhwc_debug_plan.argtypes = [i64, i64, i64, i64, ci, ci, ci, ctypes.POINTER(i64)]
+    lib.gnnhwc_debug_plan.restype = ci
     lib.gnnhwc_kernel_kind_name.argtypes = [ci]
     lib.gnnhwc_kernel_kind_name.restype = ctypes.c_char_p
     return lib

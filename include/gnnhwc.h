@@ -178,6 +178,18 @@ int gnnhwc_debug_set_spin_limit(int polls);
 int gnnhwc_debug_copy(void *dst, const void *src, size_t bytes, void *stream /* hipStream_t */);
 
 /*
+ * The tiling the multi-launch kernels would use for a problem (no counterpart in the reference, whose
+ * calc_block_params, gn_kernel.cu:37-60, is internal too); nothing is launched, no GPU is needed.  For tests of the
+ * host-side planning.  vector: 1 = 16-byte lane vectors (C must be a multiple of 16 / sizeof(dtype)), 0 = scalar
+ * kernels; backward: 0 / 1.  out[12] receives: elements per lane vector, lane vectors per row, lane vectors of a
+ * row per workgroup, chunks along C, rows per step, rows per tile, tiles per sample, most groups a chunk
+ * intersects, workgroups per launch, 1 if a compaction launch runs between producer and consumer, bytes of
+ * workspace this tiling needs, channels per group.
+ */
+int gnnhwc_debug_plan(int64_t N, int64_t R, int64_t C, int64_t G, int dtype, int vector, int backward,
+                      int64_t *out /* [12] */);
+
+/*
  * In-kernel timeline of the single-launch kernels, for tuning (no counterpart in the reference; its
  * nearest relative is the DEBUG(...) launch-parameter printf, gn_kernel.cu:13-19).  With GNNHWC_TRACE=1
  * in the environment at the first call, thread 0 of every workgroup of a single-launch kernel writes a

@@ -24,7 +24,8 @@ def test_library_exports_every_declared_symbol():
     names = _declared_functions()
     assert {"gnnhwc_fwd", "gnnhwc_fwd_add", "gnnhwc_bwd", "gnnhwc_fwd_workspace_bytes", "gnnhwc_bwd_workspace_bytes", "gnnhwc_last_error",
             "gnnhwc_version", "gnnhwc_profile_enable", "gnnhwc_profile_collect", "gnnhwc_kernel_kind_name",
-            "gnnhwc_debug_read_trace", "gnnhwc_set_resident", "gnnhwc_debug_copy", "gnnhwc_debug_set_spin_limit"} <= set(names)
+            "gnnhwc_debug_read_trace", "gnnhwc_set_resident", "gnnhwc_debug_copy", "gnnhwc_debug_set_spin_limit",
+            "gnnhwc_debug_plan"} <= set(names)
     lib = ctypes.CDLL(_cabi.LIB_PATH)
     for n in names:
         assert hasattr(lib, n), n
@@ -185,4 +186,54 @@ def test_fused_addition_operator_on_meta_tensors():
     assert gx.shape == x.shape and gt.shape == (N, C) and gt.dtype == torch.bfloat16
     with pytest.raises(RuntimeError):
         group_norm_nhwc(x, w, b, G, 1e-5, "silu", residual=mk(N, C, H, W + 1))
+
+
+def _plan(N, R, C, G, dtype, vector, backward):
+    out = (ctypes.c_int64 * 12)()
+    rc = _cabi.lib.gnnhwc_debug_plan(N, R, C, G, dtype, vector, backward, out)
+    assert rc == 0, _cabi.last_error()
+    keys = ("vec", "cv", "lpr", "nchunk", "rpi", "tile_rows", "tiles", "gmax", "nblocks", "compaction", "bytes", "D")
+    return dict(zip(keys, (int(v) for v in out)))
+
+
+def test_tiling_invariants_over_many_shapes():
+    """Host-side planning (the replacement of calc_block_params / closest_factor, gn_kernel.cu:37-60,121-128) on the
+    benchmark shapes and a seeded sample of awkward ones: the tiles cover the tensor exactly once, a workgroup's
+    lanes fit its chunk, the grid stays within the launch limits, and the workspace the public size query reports
+    holds what the tiling needs."""
+    import random
+
+    rng = random.Random(5)
+    shapes = [(1, 4096, 320, 32), (2, 1024, 640, 32), (1, 16384, 640, 32), (1, 4096, 1280, 32), (4, 16384, 320, 32),
+              (1, 262144, 128, 32), (1, 65536, 256, 32), (3, 1961, 96, 24), (8, 289, 1920, 32), (2, 2048, 256, 16),
+              (1, 1, 1, 1), (2, 5, 7, 7), (70000, 3, 8, 2), (1, 3, 4096, 1), (1, 10 ** 7, 8, 8)]
+    for _ in range(300):
+        G = rng.choice([1, 2, 3, 4, 7, 8, 16, 24, 32, 64])
+        D = rng.choice([1, 2, 3, 4, 5, 8, 10, 12, 20, 33, 40, 60, 128])
+        shapes.append((rng.randint(1, 9), rng.choice([1, 2, 7, 64, 289, 1000, 1961, 4096, 16384, 100003]), G * D, G))
+    elem = {0: 4, 1: 8, 2: 2, 3: 2}
+    for (N, R, C, G) in shapes:
+        for dtype in (0, 1, 2, 3):
+            for vector in (0, 1):
+                if vector and C % (16 // elem[dtype]) != 0:
+                    continue
+                for backward in (0, 1):
+                    p = _plan(N, R, C, G, dtype, vector, backward)
+                    ctx = (N, R, C, G, dtype, vector, backward, p)
+                    assert p["vec"] == (16 // elem[dtype] if vector else 1) and p["cv"] * p["vec"] == C, ctx
+                    assert p["D"] * G == C, ctx
+                    assert 1 <= p["lpr"] <= 256 and p["rpi"] == 256 // p["lpr"] and p["rpi"] >= 1, ctx
+                    assert (p["nchunk"] - 1) * p["lpr"] < p["cv"] <= p["nchunk"] * p["lpr"], ctx  # chunks cover the row once
+                    assert p["tile_rows"] >= 1 and p["tile_rows"] % p["rpi"] == 0 or p["tile_rows"] >= R, ctx
+                    assert (p["tiles"] - 1) * p["tile_rows"] < R <= p["tiles"] * p["tile_rows"], ctx  # tiles cover the rows once
+                    assert p["nblocks"] == N * p["tiles"] * p["nchunk"], ctx
+                    assert p["tiles"] < 2 ** 31 and p["nchunk"] <= 65535, ctx  # grid x / y limits
+                    assert 1 <= p["gmax"] <= G, ctx
+                    query = (_cabi.lib.gnnhwc_bwd_workspace_bytes if backward else _cabi.lib.gnnhwc_fwd_workspace_bytes)(N, R, C, G, dtype)
+                    assert p["bytes"] <= query, ctx
+    # a large tensor is cut into about a resident wave's worth of workgroups, not more
+    big = _plan(1, 262144, 128, 32, 2, 1, 1)
+    assert 256 <= big["nblocks"] <= 2048, big
+    out = (ctypes.c_int64 * 12)()
+    assert _cabi.lib.gnnhwc_debug_plan(1, 16, 12, 4, 3, 1, 0, out) == -1 and "vector width" in _cabi.last_error()
 
