@@ -599,28 +599,8 @@ __device__ __forceinline__ void commit_chunk_stats(const StagedStats<A> &st, con
   }
 }
 
-// gamma / beta of the lane's channels.  Issued early, next to the first data loads, so that their latency
-// is hidden behind whatever the kernel has to wait for anyway.
-template <typename A, typename PT, int VEC>
-__device__ __forceinline__ void lane_params(const LanePos &l, const void *w, const void *b, A (&gamma)[VEC],
-                                            A (&beta)[VEC]) {
-  const int c = l.cvi * VEC;
-  if (w) {
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) gamma[j] = load_param<PT, A>(w, c + j);
-  } else {
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) gamma[j] = (A)1;
-  }
-  if (b) {
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) beta[j] = load_param<PT, A>(b, c + j);
-  } else {
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) beta[j] = (A)0;
-  }
-}
-// The same without control flow, for kernels whose bulk loads are all issued up front: a load under a branch
+// gamma / beta of the lane's channels, requested early (next to the first data loads, so that their latency is
+// hidden behind whatever the kernel has to wait for anyway) and without control flow: a load under a branch
 // makes the compiler drain every outstanding load where the branch joins.  Absent parameters are read from
 // `safe` (any readable 64 bytes) and replaced by 1 / 0; c is the lane's first channel, already clamped into range.
 template <typename A, typename PT, int VEC>
