@@ -56,8 +56,51 @@ def _as_nrc(t):
     return t if t.is_contiguous() else t.contiguous()
 
 
-def _workspace(nbytes, device):
-    return torch.empty((nbytes,), dtype=torch.uint8, device=device)
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+def _current_stream_ptr(device):
+    """hipStream_t of torch's current stream on `device` (the raw getter is an order of magnitude cheaper than
+    building a torch.cuda.Stream object on every call)."""
+    if _raw_stream is not None:
+        return _raw_stream(device.index)
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+class _on_device:
+    """Makes `device` current for the C ABI call (the reference has no device guard, custom_gn.cpp:10-42); does
+    nothing when it already is, which is the usual case and keeps the context manager off the hot path."""
+
+    __slots__ = ("guard",)
+
+    def __init__(self, device):
+        self.guard = None if device.index == torch.cuda.current_device() else torch.cuda.device(device)
+
+    def __enter__(self):
+        if self.guard is not None:
+            self.guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self.guard is not None:
+            self.guard.__exit__(*exc)
+        return False
+
+
+_workspaces = {}
+
+
+def _workspace(nbytes, device, stream_ptr):
+    """Scratch memory for one call.  Calls on one stream follow each other, so they can share one buffer per
+    (device, stream), grown on demand; while the stream is recording a graph the buffer comes from the allocator
+    instead (it then belongs to the graph's own memory pool, like every other tensor of the capture)."""
+    if torch.cuda.is_current_stream_capturing():
+        return torch.empty((nbytes,), dtype=torch.uint8, device=device)
+    key = (device.index, stream_ptr)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty((max(nbytes, 1 << 20),), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
 
 
 def gn_nhwc_fwd(X, weight, bias, G, eps, act_fn_option):
@@ -80,16 +123,17 @@ def gn_nhwc_fwd(X, weight, bias, G, eps, act_fn_option):
     means = torch.empty((N, G), dtype=sdtype, device=X.device)
     rstds = torch.empty((N, G), dtype=sdtype, device=X.device)
     lib = _cabi.lib
-    with torch.cuda.device(X.device):
+    with _on_device(X.device):
         nbytes = lib.gnnhwc_fwd_workspace_bytes(N, R, C, G, dt)
         if nbytes == 0:
             raise RuntimeError("gnop::fwd: " + _cabi.last_error())
-        ws = _workspace(nbytes, X.device)
+        stream = _current_stream_ptr(X.device)
+        ws = _workspace(nbytes, X.device, stream)
         rc = lib.gnnhwc_fwd(
             X_nrc.data_ptr(), weight.contiguous().data_ptr(), bias.contiguous().data_ptr(),
             Y.data_ptr(), means.data_ptr(), rstds.data_ptr(),
             N, R, C, G, float(eps), int(act_fn_option), dt, pdt, _DTYPE_CODE[sdtype],
-            ws.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream)
+            ws.data_ptr(), ws.numel(), stream)
     _cabi.check(rc, "gnop::fwd")
     return Y.permute(0, 2, 1), means, rstds
 
@@ -117,17 +161,18 @@ def gn_nhwc_bwd(dy, X, weight, bias, means, rstds, G, act_fn_option):
     dweight = torch.empty((C,), dtype=weight.dtype, device=X.device)
     dbias = torch.empty((C,), dtype=weight.dtype, device=X.device)
     lib = _cabi.lib
-    with torch.cuda.device(X.device):
+    with _on_device(X.device):
         nbytes = lib.gnnhwc_bwd_workspace_bytes(N, R, C, G, dt)
         if nbytes == 0:
             raise RuntimeError("gnop::bwd: " + _cabi.last_error())
-        ws = _workspace(nbytes, X.device)
+        stream = _current_stream_ptr(X.device)
+        ws = _workspace(nbytes, X.device, stream)
         rc = lib.gnnhwc_bwd(
             dy_nrc.data_ptr(), X_nrc.data_ptr(), weight.contiguous().data_ptr(), bias.contiguous().data_ptr(),
             means.contiguous().data_ptr(), rstds.contiguous().data_ptr(),
             dX.data_ptr(), dweight.data_ptr(), dbias.data_ptr(),
             N, R, C, G, int(act_fn_option), dt, pdt, sdt,
-            ws.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream)
+            ws.data_ptr(), ws.numel(), stream)
     _cabi.check(rc, "gnop::bwd")
     return dX.permute(0, 2, 1), dweight, dbias
 
@@ -170,17 +215,18 @@ def gn_nhwc_fwd_add(X, residual, channel_bias, weight, bias, G, eps, act_fn_opti
     means = torch.empty((N, G), dtype=sdtype, device=X.device)
     rstds = torch.empty((N, G), dtype=sdtype, device=X.device)
     lib = _cabi.lib
-    with torch.cuda.device(X.device):
+    with _on_device(X.device):
         nbytes = lib.gnnhwc_fwd_workspace_bytes(N, R, C, G, dt)
         if nbytes == 0:
             raise RuntimeError("gnop::fwd_add: " + _cabi.last_error())
-        ws = _workspace(nbytes, X.device)
+        stream = _current_stream_ptr(X.device)
+        ws = _workspace(nbytes, X.device, stream)
         rc = lib.gnnhwc_fwd_add(
             X_nrc.data_ptr(), res_ptr, cb_ptr, S.data_ptr() if return_sum else None,
             weight.contiguous().data_ptr(), bias.contiguous().data_ptr(),
             Y.data_ptr(), means.data_ptr(), rstds.data_ptr(),
             N, R, C, G, float(eps), int(act_fn_option), dt, pdt, _DTYPE_CODE[sdtype], cb_dt,
-            ws.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream)
+            ws.data_ptr(), ws.numel(), stream)
     _cabi.check(rc, "gnop::fwd_add")
     return Y.permute(0, 2, 1), S.permute(0, 2, 1), means, rstds
 
@@ -332,7 +378,9 @@ class GN_NHWC_Func(torch.autograd.Function):
         for d in X.shape[2:]:
             R *= d
         X_flat = X.view(X.shape[0], X.shape[1], R)  # explicit R: "-1" is ambiguous for an empty batch
-        X_out, means, rstds = torch.ops.gnop.fwd(X_flat, weight, bias, G, eps, activation)
+        # the operator's own implementation, called directly: going through torch.ops.gnop.fwd would add the
+        # dispatcher and its autograd wrapper to every call, and this Function already is the autograd formula
+        X_out, means, rstds = gn_nhwc_fwd(X_flat, weight, bias, G, eps, activation)
         ctx.save_for_backward(X_flat, weight, bias, means, rstds)
         ctx.G = G
         ctx.activation = activation
@@ -348,7 +396,7 @@ class GN_NHWC_Func(torch.autograd.Function):
         dy_last = dy.permute(0, *range(2, nd), 1).contiguous()
         dy_flat = dy_last.view(X_flat.shape[0], X_flat.shape[2], X_flat.shape[1]).permute(0, 2, 1)
         assert dy_flat.stride() == X_flat.stride() or X_flat.numel() == 0 or 1 in X_flat.shape
-        dx, dgamma, dbeta = torch.ops.gnop.bwd(dy_flat, X_flat, weight, bias, means, rstds, ctx.G, ctx.activation)
+        dx, dgamma, dbeta = gn_nhwc_bwd(dy_flat, X_flat, weight, bias, means, rstds, ctx.G, ctx.activation)
         return dx.view(ctx.x_shape), dgamma, dbeta, None, None, None
 
 
