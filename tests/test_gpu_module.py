@@ -681,3 +681,29 @@ def test_more_than_two_to_the_31_elements(device):
             # every element of dx carries a bf16 rounding error of relative size 2^-9 with random sign
             assert float(total) <= float(scale) * 2.0 ** -9 * 8 / (R * D) ** 0.5
     assert _device_err(dw, dw_sum) <= 2.0 ** -7 and _device_err(db, db_sum) <= 2.0 ** -7
+
+
+@pytest.mark.gpu
+def test_module_on_two_streams(device):
+    """The Python surface keeps one scratch buffer per (device, stream): the same module called on two torch streams
+    with no synchronisation in between gives, on each, the results of the same calls made alone."""
+    gen = torch.Generator().manual_seed(91)
+    m = GN_NHWC(32, 640, activation="silu").to(device=device, dtype=torch.bfloat16)
+    with torch.no_grad():
+        m.weight.copy_((torch.rand(640, generator=gen) + 0.5).to(torch.bfloat16))
+        m.bias.copy_((0.1 * torch.randn(640, generator=gen)).to(torch.bfloat16))
+    xs = [channels_last_like((1, 640, 48, 48), torch.bfloat16, device, gen, 1.0 + i, 0.3 * i) for i in range(2)]
+    with torch.no_grad():
+        want = [m(x).clone() for x in xs]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    got = [[], []]
+    with torch.no_grad():
+        for _ in range(25):
+            for i, s in enumerate(streams):
+                with torch.cuda.stream(s):
+                    got[i].append(m(xs[i]))
+    torch.cuda.synchronize()
+    for i in range(2):
+        for y in got[i]:
+            assert torch.equal(y, want[i])
