@@ -51,6 +51,9 @@ def parse_args():
     ap.add_argument("--fused-add", action="store_true",
                     help="also time gnnhwc_fwd_add (residual + sum output fused into the forward) against an elementwise "
                          "addition followed by gnnhwc_fwd, per shape (reported under 'fused_add')")
+    ap.add_argument("--nchw", action="store_true",
+                    help="also time the channels-first entry points on the same shapes against torch's GroupNorm + activation "
+                         "on channels-first tensors (reported under 'channels_first')")
     ap.add_argument("--counter-workload", action="store_true",
                     help="no timing: one 256 MiB plain copy (calibration) and a few fwd+bwd calls per shape, for a rocprofv3 --pmc run")
     return ap.parse_args()
@@ -406,6 +409,76 @@ def fused_add_table(names, device, steps, warmup):
     return out
 
 
+def nchw_table(names, device, steps, warmup):
+    """gnnhwc_fwd_nchw / gnnhwc_bwd_nchw (two launches forward, three backward; algorithmic bytes 2 S / 3 S as for the
+    channels-last path) against what the reference does with channels-first input: torch's GroupNorm followed by the
+    activation, and their autograd backward."""
+    import torch
+    import torch.nn.functional as F
+    from tests import configs
+    from tests.gpu_harness import DT_CODE
+
+    acts = {"identity": lambda t: t, "relu": F.relu, "silu": F.silu, "gelu": F.gelu,
+            "gelu_tanh": lambda t: F.gelu(t, approximate="tanh")}
+    out = {}
+    for n in names:
+        cfg = configs.CONFIGS[n]
+        p = Problem(cfg, device)
+        b = p.sets[0]
+        x = b["x"].permute(0, 2, 1).contiguous()   # (N, C, R)
+        dy = b["dy"].permute(0, 2, 1).contiguous()
+        y, dx = torch.empty_like(x), torch.empty_like(x)
+        lib = p.lib
+        nb = max(lib.gnnhwc_nchw_workspace_bytes(p.N, p.C, p.R, p.G, p.dt, 0), lib.gnnhwc_nchw_workspace_bytes(p.N, p.C, p.R, p.G, p.dt, 1))
+        ws = torch.empty((nb,), dtype=torch.uint8, device=device)
+        stream_of = lambda: torch.cuda.current_stream().cuda_stream  # noqa: E731
+
+        def fwd():
+            rc = lib.gnnhwc_fwd_nchw(x.data_ptr(), p.w.data_ptr(), p.b.data_ptr(), y.data_ptr(), p.mean.data_ptr(), p.rstd.data_ptr(),
+                                     p.N, p.C, p.R, p.G, 1e-5, p.act, p.dt, p.dt, p.sdt, ws.data_ptr(), nb, stream_of())
+            if rc != 0:
+                raise RuntimeError(lib.gnnhwc_last_error().decode())
+
+        def bwd():
+            rc = lib.gnnhwc_bwd_nchw(dy.data_ptr(), x.data_ptr(), p.w.data_ptr(), p.b.data_ptr(), p.mean.data_ptr(), p.rstd.data_ptr(),
+                                     dx.data_ptr(), p.dw.data_ptr(), p.db.data_ptr(), p.N, p.C, p.R, p.G, p.act, p.dt, p.dt, p.sdt,
+                                     ws.data_ptr(), nb, stream_of())
+            if rc != 0:
+                raise RuntimeError(lib.gnnhwc_last_error().decode())
+
+        xt = x.view(p.N, p.C, p.R, 1).clone().requires_grad_()
+        wt, bt = p.w.clone().requires_grad_(), p.b.clone().requires_grad_()
+        act = acts[cfg.act]
+        dyt = dy.view(p.N, p.C, p.R, 1)
+
+        def torch_fwd():
+            with torch.no_grad():
+                act(F.group_norm(xt, p.G, wt, bt, 1e-5))
+
+        def torch_fwd_bwd():
+            yt = act(F.group_norm(xt, p.G, wt, bt, 1e-5))
+            torch.autograd.grad(yt, (xt, wt, bt), dyt)
+
+        def ours_fwd_bwd():
+            fwd()
+            bwd()
+
+        r = {}
+        for key, fn, streams in (("fwd", fwd, 2), ("fwd_bwd", ours_fwd_bwd, 5), ("torch_fwd", torch_fwd, 2), ("torch_fwd_bwd", torch_fwd_bwd, 5)):
+            if key.endswith("bwd") and not p.bwd:
+                continue
+            t = min(time_region(fn, steps, warmup, False) for _ in range(3)) / steps
+            r[key + "_us"] = round(t * 1e6, 3)
+            r[key + "_gbps"] = round(streams * p.S / t / 1e9, 1)
+        r["fwd_speedup_over_torch"] = round(r["torch_fwd_us"] / r["fwd_us"], 3)
+        if p.bwd:
+            r["fwd_bwd_speedup_over_torch"] = round(r["torch_fwd_bwd_us"] / r["fwd_bwd_us"], 3)
+        out[n] = r
+        del p
+        torch.cuda.empty_cache()
+    return out
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -532,6 +605,8 @@ def main():
         "roofline": roofline,
         "shapes": shapes,
     }
+    if args.nchw:
+        line["channels_first"] = nchw_table(head_names, device, max(20, args.steps // 2), args.warmup)
     if args.fused_add:
         line["fused_add"] = fused_add_table(head_names, device, max(20, args.steps // 2), args.warmup)
     if not args.no_cpu_baseline:

@@ -602,6 +602,90 @@ int gnnhwc_debug_copy(void *dst, const void *src, size_t bytes, void *stream) {
   return GNNHWC_OK;
 }
 
+// ---- channels-first layout -----------------------------------------------------------------------------------
+static int nchw_vec(int dtype, int64_t R, const void *a, const void *b, const void *c) {
+  const int vec = 16 / elem_size(dtype);
+  return (R % vec == 0 && aligned16(a) && aligned16(b) && aligned16(c)) ? vec : 1;
+}
+size_t gnnhwc_nchw_workspace_bytes(int64_t N, int64_t C, int64_t R, int64_t G, int dtype, int backward) {
+  if (check_shape(N, R, C, G, dtype) != GNNHWC_OK) return 0;
+  if (N == 0 || R == 0) return 256;
+  // the scalar kernels have the most chunks per row: enough for either path
+  return align_up(nchw_workspace_elems(N, C, R, 1, backward != 0) * acc_size(dtype), 256);
+}
+static int nchw_call(NchwArgs &a, int dtype, void *workspace, size_t workspace_bytes, const char *what) {
+  const size_t need = gnnhwc_nchw_workspace_bytes(a.N, a.C, a.R, a.G, dtype, a.backward ? 1 : 0);
+  if (!workspace || !aligned16(workspace) || workspace_bytes < need)
+    return fail(GNNHWC_ERR_WORKSPACE, "%s workspace must be 16-byte aligned and at least %zu bytes (got %p, %zu bytes)", what,
+                need, workspace, workspace_bytes);
+  const int vec = a.vector ? 16 / (int)elem_size(dtype) : 1;
+  const int64_t chunks = (a.R + nchw_chunk_len(vec) - 1) / nchw_chunk_len(vec);
+  if ((double)a.N * (double)a.C * (double)chunks / 4.0 > 2.0e9)
+    return fail(GNNHWC_ERR_INVALID_ARGUMENT, "%s: too many rows for one launch (N C = %lld)", what, (long long)(a.N * a.C));
+  a.ws = workspace;
+  hipError_t e;
+  switch (dtype) {
+    case GN_F32: e = launch_nchw_f32(a); break;
+    case GN_F64: e = launch_nchw_f64(a); break;
+    case GN_F16: e = launch_nchw_f16(a); break;
+    default: e = launch_nchw_bf16(a); break;
+  }
+  if (e != hipSuccess) return fail(GNNHWC_ERR_LAUNCH, "%s launch failed: %s", what, hipGetErrorString(e));
+  return GNNHWC_OK;
+}
+
+int gnnhwc_fwd_nchw(const void *x, const void *weight, const void *bias, void *y, void *mean, void *rstd, int64_t N,
+                    int64_t C, int64_t R, int64_t G, double eps, int act, int dtype, int param_dtype, int stats_dtype,
+                    void *workspace, size_t workspace_bytes, void *stream) {
+  int rc = check_shape(N, R, C, G, dtype);
+  if (rc != GNNHWC_OK) return rc;
+  rc = check_dtypes(dtype, param_dtype, stats_dtype);
+  if (rc != GNNHWC_OK) return rc;
+  if (act < GN_ACT_IDENTITY || act > GN_ACT_GELU_TANH)
+    return fail(GNNHWC_ERR_INVALID_ARGUMENT, "unknown activation code %d", act);
+  if (N == 0 || R == 0) return GNNHWC_OK;
+  if (!x || !y) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "x and y must not be null");
+  NchwArgs a = {};
+  a.backward = false;
+  a.vector = nchw_vec(dtype, R, x, y, nullptr) > 1;
+  a.x = x; a.w = weight; a.b = bias; a.y = y; a.mean_out = mean; a.rstd_out = rstd;
+  a.N = N; a.C = C; a.R = R; a.G = G;
+  a.eps = eps; a.act = act; a.pdtype = param_dtype; a.sdtype = stats_dtype;
+  a.stream = (hipStream_t)stream;
+  return nchw_call(a, dtype, workspace, workspace_bytes, "channels-first forward");
+}
+
+int gnnhwc_bwd_nchw(const void *dy, const void *x, const void *weight, const void *bias, const void *mean, const void *rstd,
+                    void *dx, void *dweight, void *dbias, int64_t N, int64_t C, int64_t R, int64_t G, int act, int dtype,
+                    int param_dtype, int stats_dtype, void *workspace, size_t workspace_bytes, void *stream) {
+  int rc = check_shape(N, R, C, G, dtype);
+  if (rc != GNNHWC_OK) return rc;
+  rc = check_dtypes(dtype, param_dtype, stats_dtype);
+  if (rc != GNNHWC_OK) return rc;
+  if (act < GN_ACT_IDENTITY || act > GN_ACT_GELU_TANH)
+    return fail(GNNHWC_ERR_INVALID_ARGUMENT, "unknown activation code %d", act);
+  if (N == 0 || R == 0) {
+    const unsigned grid = (unsigned)((C + 255) / 256);
+    if (dweight) hipLaunchKernelGGL(fill_zero_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, dweight, C, param_dtype);
+    if (dbias) hipLaunchKernelGGL(fill_zero_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, dbias, C, param_dtype);
+    const hipError_t e0 = hipGetLastError();
+    if (e0 != hipSuccess) return fail(GNNHWC_ERR_LAUNCH, "backward launch failed: %s", hipGetErrorString(e0));
+    return GNNHWC_OK;
+  }
+  if (!dy || !x || !mean || !rstd || !dx)
+    return fail(GNNHWC_ERR_INVALID_ARGUMENT, "dy, x, mean, rstd and dx must not be null");
+  if (N * G > 0x7fffffffLL) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "N * G too large");
+  NchwArgs a = {};
+  a.backward = true;
+  a.vector = nchw_vec(dtype, R, x, dy, dx) > 1;
+  a.x = x; a.dy = dy; a.w = weight; a.b = bias; a.mean = mean; a.rstd = rstd;
+  a.dx = dx; a.dw = dweight; a.db = dbias;
+  a.N = N; a.C = C; a.R = R; a.G = G;
+  a.eps = 0.0; a.act = act; a.pdtype = param_dtype; a.sdtype = stats_dtype;
+  a.stream = (hipStream_t)stream;
+  return nchw_call(a, dtype, workspace, workspace_bytes, "channels-first backward");
+}
+
 int gnnhwc_debug_plan(int64_t N, int64_t R, int64_t C, int64_t G, int dtype, int vector, int backward, int64_t *out) {
   if (!out) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "null output array");
   const int rc = check_shape(N, R, C, G, dtype);
@@ -621,7 +705,8 @@ int gnnhwc_debug_plan(int64_t N, int64_t R, int64_t C, int64_t G, int dtype, int
 const char *gnnhwc_kernel_kind_name(int kind) {
   static const char *names[GNNHWC_NUM_KERNEL_KINDS] = {"fwd_stats", "fwd_stats_compact", "fwd_apply", "bwd_reduce",
                                                        "bwd_compact", "bwd_dx", "fused_fwd", "fused_bwd", "copy",
-                                                       "fwd_add", "fused_fwd_add"};
+                                                       "fwd_add", "fused_fwd_add",
+                                                       "nchw_stats", "nchw_apply", "nchw_bwd_reduce", "nchw_bwd_dx", "nchw_dwdb"};
   return (kind >= 0 && kind < GNNHWC_NUM_KERNEL_KINDS) ? names[kind] : "";
 }
 

@@ -21,6 +21,11 @@ enum KernelKind {
   kKindCopy = 8,
   kKindAdd = 9,        // elementwise pre-addition of the multi-launch fused-addition forward
   kKindFusedFwdAdd = 10,  // single-launch forward with the pre-addition fused in
+  kKindNchwStats = 11,    // channels-first layout: forward statistics, forward apply, backward reduce, backward dx,
+  kKindNchwApply = 12,    // dgamma / dbeta
+  kKindNchwBwdReduce = 13,
+  kKindNchwBwdDx = 14,
+  kKindNchwDwDb = 15,
   kNumKinds = 9
 };
 
@@ -43,6 +48,26 @@ struct BwdArgs {
   hipStream_t stream;
   Plan plan;
 };
+
+// One call on a channels-first tensor (N, C, R contiguous): forward (x -> y, mean_out, rstd_out) or backward
+// (dy, x, mean, rstd -> dx, dw, db).
+struct NchwArgs {
+  bool backward, vector;  // vector: 16-byte lane vectors (R a multiple of the vector width, aligned pointers)
+  const void *x, *dy, *w, *b, *mean, *rstd;
+  void *y, *dx, *dw, *db, *mean_out, *rstd_out;
+  int64_t N, C, R, G;
+  double eps;
+  int act, pdtype, sdtype;
+  void *ws;
+  hipStream_t stream;
+};
+// Elements of one chunk of a channel row: 64 lanes x vec elements x 4 lane vectors (kNchwUnroll in gn_nchw.h).
+inline int nchw_chunk_len(int vec) { return 64 * vec * 4; }
+// Accumulation-type elements of workspace: 3 planes forward, 2 backward, of [N * C][chunks].
+inline size_t nchw_workspace_elems(int64_t N, int64_t C, int64_t R, int vec, bool backward) {
+  const int64_t chunks = (R + nchw_chunk_len(vec) - 1) / nchw_chunk_len(vec);
+  return (size_t)(backward ? 2 : 3) * (size_t)(N * C * chunks);
+}
 
 // Workspace layout, in elements of the accumulation type (float, or double for f64 data).
 struct FwdWorkspace {
@@ -165,5 +190,9 @@ hipError_t launch_bwd_f32(const BwdArgs &a);
 hipError_t launch_bwd_f64(const BwdArgs &a);
 hipError_t launch_bwd_f16(const BwdArgs &a);
 hipError_t launch_bwd_bf16(const BwdArgs &a);
+hipError_t launch_nchw_f32(const NchwArgs &a);
+hipError_t launch_nchw_f64(const NchwArgs &a);
+hipError_t launch_nchw_f16(const NchwArgs &a);
+hipError_t launch_nchw_bf16(const NchwArgs &a);
 
 }  // namespace gn

@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(_CSRC, "libgnnhwc_hip.so")
 
 # dtype / activation codes of include/gnnhwc.h
 F32, F64, F16, BF16 = 0, 1, 2, 3
-NUM_KERNEL_KINDS = 11
+NUM_KERNEL_KINDS = 16
 
 SYMBOLS = (
     "gnnhwc_version",
@@ -22,6 +22,9 @@ SYMBOLS = (
     "gnnhwc_fwd",
     "gnnhwc_fwd_add",
     "gnnhwc_bwd",
+    "gnnhwc_nchw_workspace_bytes",
+    "gnnhwc_fwd_nchw",
+    "gnnhwc_bwd_nchw",
     "gnnhwc_profile_enable",
     "gnnhwc_profile_collect",
     "gnnhwc_kernel_kind_name",
@@ -54,6 +57,12 @@ def _load():
     lib.gnnhwc_fwd_add.restype = ci
     lib.gnnhwc_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, ci, ci, ci, ci, vp, sz, vp]
     lib.gnnhwc_bwd.restype = ci
+    lib.gnnhwc_nchw_workspace_bytes.argtypes = [i64, i64, i64, i64, ci, ci]
+    lib.gnnhwc_nchw_workspace_bytes.restype = sz
+    lib.gnnhwc_fwd_nchw.argtypes = list(lib.gnnhwc_fwd.argtypes)
+    lib.gnnhwc_fwd_nchw.restype = ci
+    lib.gnnhwc_bwd_nchw.argtypes = list(lib.gnnhwc_bwd.argtypes)
+    lib.gnnhwc_bwd_nchw.restype = ci
     lib.gnnhwc_profile_enable.argtypes = [ci]
     lib.gnnhwc_profile_enable.restype = ci
     lib.gnnhwc_profile_collect.argtypes = [ctypes.POINTER(i64), ctypes.POINTER(dbl)]

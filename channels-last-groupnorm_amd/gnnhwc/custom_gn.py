@@ -177,6 +177,81 @@ def gn_nhwc_bwd(dy, X, weight, bias, means, rstds, G, act_fn_option):
     return dX.permute(0, 2, 1), dweight, dbias
 
 
+def gn_nchw_fwd(X, weight, bias, G, eps, act_fn_option):
+    """gnop::fwd_nchw (no counterpart in the reference, which hands channels-first input to torch,
+    custom_gn.py:75-79): X is (N, C, R) contiguous.  Returns (Y contiguous like X, means, rstds)."""
+    _check_device(X, "X")
+    _check_device(weight, "weight")
+    _check_device(bias, "bias")
+    if X.dim() != 3:
+        raise RuntimeError("gnop::fwd_nchw expects X of shape (N, C, R), got %s" % (tuple(X.shape),))
+    N, C, R = X.shape
+    dt = _dtype_code(X, "X")
+    pdt = _dtype_code(weight, "weight")
+    if bias.dtype != weight.dtype:
+        raise RuntimeError("weight and bias must have the same dtype (%s vs %s)" % (weight.dtype, bias.dtype))
+    if weight.numel() != C or bias.numel() != C:
+        raise RuntimeError("weight and bias must have %d elements" % C)
+    X = X.contiguous()
+    Y = torch.empty_like(X)
+    sdtype = _stats_dtype(X.dtype)
+    means = torch.empty((N, G), dtype=sdtype, device=X.device)
+    rstds = torch.empty((N, G), dtype=sdtype, device=X.device)
+    lib = _cabi.lib
+    with _on_device(X.device):
+        nbytes = lib.gnnhwc_nchw_workspace_bytes(N, C, R, G, dt, 0)
+        if nbytes == 0:
+            raise RuntimeError("gnop::fwd_nchw: " + _cabi.last_error())
+        stream = _current_stream_ptr(X.device)
+        ws = _workspace(nbytes, X.device, stream)
+        rc = lib.gnnhwc_fwd_nchw(
+            X.data_ptr(), weight.contiguous().data_ptr(), bias.contiguous().data_ptr(),
+            Y.data_ptr(), means.data_ptr(), rstds.data_ptr(),
+            N, C, R, G, float(eps), int(act_fn_option), dt, pdt, _DTYPE_CODE[sdtype],
+            ws.data_ptr(), ws.numel(), stream)
+    _cabi.check(rc, "gnop::fwd_nchw")
+    return Y, means, rstds
+
+
+def gn_nchw_bwd(dy, X, weight, bias, means, rstds, G, act_fn_option):
+    """gnop::bwd_nchw: dy, X (N, C, R) contiguous.  Returns (dX, dweight, dbias)."""
+    for t, name in ((dy, "dy"), (X, "X"), (weight, "weight"), (bias, "bias"), (means, "means"), (rstds, "rstds")):
+        _check_device(t, name)
+    if X.dim() != 3 or dy.shape != X.shape:
+        raise RuntimeError("gnop::bwd_nchw expects dy and X of the same shape (N, C, R), got %s and %s"
+                           % (tuple(dy.shape), tuple(X.shape)))
+    N, C, R = X.shape
+    dt = _dtype_code(X, "X")
+    pdt = _dtype_code(weight, "weight")
+    sdt = _dtype_code(means, "means")
+    if dy.dtype != X.dtype:
+        raise RuntimeError("dy and X must have the same dtype (%s vs %s)" % (dy.dtype, X.dtype))
+    if rstds.dtype != means.dtype or bias.dtype != weight.dtype:
+        raise RuntimeError("means/rstds and weight/bias must pairwise share a dtype")
+    if means.numel() != N * G or rstds.numel() != N * G:
+        raise RuntimeError("means and rstds must have N*G = %d elements" % (N * G))
+    X = X.contiguous()
+    dy = dy.contiguous()
+    dX = torch.empty_like(X)
+    dweight = torch.empty((C,), dtype=weight.dtype, device=X.device)
+    dbias = torch.empty((C,), dtype=weight.dtype, device=X.device)
+    lib = _cabi.lib
+    with _on_device(X.device):
+        nbytes = lib.gnnhwc_nchw_workspace_bytes(N, C, R, G, dt, 1)
+        if nbytes == 0:
+            raise RuntimeError("gnop::bwd_nchw: " + _cabi.last_error())
+        stream = _current_stream_ptr(X.device)
+        ws = _workspace(nbytes, X.device, stream)
+        rc = lib.gnnhwc_bwd_nchw(
+            dy.data_ptr(), X.data_ptr(), weight.contiguous().data_ptr(), bias.contiguous().data_ptr(),
+            means.contiguous().data_ptr(), rstds.contiguous().data_ptr(),
+            dX.data_ptr(), dweight.data_ptr(), dbias.data_ptr(),
+            N, C, R, G, int(act_fn_option), dt, pdt, sdt,
+            ws.data_ptr(), ws.numel(), stream)
+    _cabi.check(rc, "gnop::bwd_nchw")
+    return dX, dweight, dbias
+
+
 def gn_nhwc_fwd_add(X, residual, channel_bias, weight, bias, G, eps, act_fn_option, return_sum):
     """gnop::fwd_add (no counterpart in the reference): gnop::fwd of S = X + residual + channel_bias[:, :, None],
     with the additions done inside the kernel.  X, residual: (N, C, R) channels-last views; channel_bias: (N, C).
@@ -240,6 +315,11 @@ _op_lib.define("bwd(Tensor dy, Tensor X, Tensor weight, Tensor bias, Tensor mean
                "int act_fn_option) -> (Tensor, Tensor, Tensor)")
 _op_lib.define("fwd_add(Tensor X, Tensor? residual, Tensor? channel_bias, Tensor weight, Tensor bias, int G, float eps, "
                "int act_fn_option, bool return_sum) -> (Tensor, Tensor, Tensor, Tensor)")
+_op_lib.define("fwd_nchw(Tensor X, Tensor weight, Tensor bias, int G, float eps, int act_fn_option) -> (Tensor, Tensor, Tensor)")
+_op_lib.define("bwd_nchw(Tensor dy, Tensor X, Tensor weight, Tensor bias, Tensor means, Tensor rstds, int G, "
+               "int act_fn_option) -> (Tensor, Tensor, Tensor)")
+_op_lib.impl("fwd_nchw", gn_nchw_fwd, "CompositeExplicitAutograd")
+_op_lib.impl("bwd_nchw", gn_nchw_bwd, "CompositeExplicitAutograd")
 _op_lib.impl("fwd", gn_nhwc_fwd, "CompositeExplicitAutograd")
 _op_lib.impl("fwd_add", gn_nhwc_fwd_add, "CompositeExplicitAutograd")
 _op_lib.impl("bwd", gn_nhwc_bwd, "CompositeExplicitAutograd")
@@ -272,6 +352,23 @@ def _fwd_add_meta(X, residual, channel_bias, weight, bias, G, eps, act_fn_option
 _op_lib.impl("fwd", _fwd_meta, "Meta")
 _op_lib.impl("bwd", _bwd_meta, "Meta")
 _op_lib.impl("fwd_add", _fwd_add_meta, "Meta")
+
+
+def _fwd_nchw_meta(X, weight, bias, G, eps, act_fn_option):
+    N = X.shape[0]
+    sdtype = _stats_dtype(X.dtype)
+    return (torch.empty(X.shape, dtype=X.dtype, device=X.device), torch.empty((N, G), dtype=sdtype, device=X.device),
+            torch.empty((N, G), dtype=sdtype, device=X.device))
+
+
+def _bwd_nchw_meta(dy, X, weight, bias, means, rstds, G, act_fn_option):
+    C = X.shape[1]
+    return (torch.empty(X.shape, dtype=X.dtype, device=X.device), torch.empty((C,), dtype=weight.dtype, device=X.device),
+            torch.empty((C,), dtype=weight.dtype, device=X.device))
+
+
+_op_lib.impl("fwd_nchw", _fwd_nchw_meta, "Meta")
+_op_lib.impl("bwd_nchw", _bwd_nchw_meta, "Meta")
 
 
 def _fwd_setup_context(ctx, inputs, output):
@@ -400,6 +497,32 @@ class GN_NHWC_Func(torch.autograd.Function):
         return dx.view(ctx.x_shape), dgamma, dbeta, None, None, None
 
 
+class GN_NCHW_Func(torch.autograd.Function):
+    """The same contract as GN_NHWC_Func for contiguous channels-first input (no counterpart in the reference,
+    which lets torch handle that layout, custom_gn.py:75-79): apply(X, weight, bias, G, eps, activation_code) -> Y
+    contiguous with X's shape."""
+
+    @staticmethod
+    def forward(ctx, X, weight, bias, G, eps, activation):
+        ctx.x_shape = X.shape
+        R = 1
+        for d in X.shape[2:]:
+            R *= d
+        X_flat = X.contiguous().view(X.shape[0], X.shape[1], R)
+        Y, means, rstds = gn_nchw_fwd(X_flat, weight, bias, G, eps, activation)
+        ctx.save_for_backward(X_flat, weight, bias, means, rstds)
+        ctx.G = G
+        ctx.activation = activation
+        return Y.view(ctx.x_shape)
+
+    @staticmethod
+    def backward(ctx, dy):
+        X_flat, weight, bias, means, rstds = ctx.saved_tensors
+        dy_flat = dy.contiguous().view(X_flat.shape)
+        dx, dgamma, dbeta = gn_nchw_bwd(dy_flat, X_flat, weight, bias, means, rstds, ctx.G, ctx.activation)
+        return dx.view(ctx.x_shape), dgamma, dbeta, None, None, None
+
+
 _TORCH_ACTIVATIONS = (
     lambda t: t,
     F.relu,
@@ -426,12 +549,19 @@ class GN_NHWC(nn.GroupNorm):
             x = x.permute(0, *range(2, nd), 1).contiguous().permute(0, nd - 1, *range(1, nd - 1))
             run = GN_NHWC_Func.apply
         else:
-            # channels-first input: torch's own GroupNorm, then the activation (custom_gn.py:75-79)
+            # channels-first input: the reference hands it to torch's GroupNorm and applies the activation in a
+            # second pass (custom_gn.py:75-79); the same result (contiguous output) comes from the channels-first
+            # kernels here, with the activation fused
             x = x.contiguous()
-            act = _TORCH_ACTIVATIONS[self.act_code]
+            if x.is_cuda:
+                run = GN_NCHW_Func.apply
+            else:
+                # not a device tensor: exactly the reference's expression (its channels-first path never reaches a
+                # kernel, so it also serves host tensors)
+                act = _TORCH_ACTIVATIONS[self.act_code]
 
-            def run(t, w, b, g, eps, _code):
-                return act(F.group_norm(t, g, w, b, eps))
+                def run(t, w, b, g, eps, _code):
+                    return act(F.group_norm(t, g, w, b, eps))
 
         if self.affine:
             w, b = self.weight, self.bias

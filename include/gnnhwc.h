@@ -130,6 +130,27 @@ int gnnhwc_bwd(const void *dy, const void *x, const void *weight, const void *bi
                void *workspace, size_t workspace_bytes, void *stream /* hipStream_t */);
 
 /*
+ * Channels-first layout: x, y, dy, dx are (N, C, R) contiguous, R fastest.  The reference has no kernel for it:
+ * GN_NHWC.forward hands such input to torch's GroupNorm and applies the activation in a second pass
+ * (custom_gn.py:75-79); these entry points give the same results with the activation fused (forward: two launches,
+ * x read twice; backward: three).  Arguments, dtypes, NULL conventions and errors are those of gnnhwc_fwd /
+ * gnnhwc_bwd, except that C comes before R; y may alias x.  Workspace: gnnhwc_nchw_workspace_bytes.
+ */
+size_t gnnhwc_nchw_workspace_bytes(int64_t N, int64_t C, int64_t R, int64_t G, int dtype, int backward);
+int gnnhwc_fwd_nchw(const void *x, const void *weight, const void *bias,
+                    void *y, void *mean, void *rstd,
+                    int64_t N, int64_t C, int64_t R, int64_t G,
+                    double eps, int act,
+                    int dtype, int param_dtype, int stats_dtype,
+                    void *workspace, size_t workspace_bytes, void *stream /* hipStream_t */);
+int gnnhwc_bwd_nchw(const void *dy, const void *x, const void *weight, const void *bias,
+                    const void *mean, const void *rstd,
+                    void *dx, void *dweight, void *dbias,
+                    int64_t N, int64_t C, int64_t R, int64_t G, int act,
+                    int dtype, int param_dtype, int stats_dtype,
+                    void *workspace, size_t workspace_bytes, void *stream /* hipStream_t */);
+
+/*
  * Kernel selection (no counterpart in the reference).  By default a problem whose tensors fit in the
  * register files of one launch is run by the single-launch kernels (x and dy are read from memory once;
  * workgroups exchange partial results while resident), anything else by the multi-launch streaming
@@ -151,9 +172,10 @@ int gnnhwc_set_resident(int on);
  * the last collect, then clears the record.  Kinds: 0 fwd statistics, 1 fwd statistics compaction
  * (many row tiles only), 2 fwd apply, 3 bwd reduce, 4 bwd compaction (many row tiles only), 5 bwd dx,
  * 6 single-launch fwd, 7 single-launch bwd, 8 the plain copy of gnnhwc_debug_copy, 9 the elementwise pre-addition
- * of gnnhwc_fwd_add's multi-launch form, 10 single-launch fwd with the pre-addition fused in.
+ * of gnnhwc_fwd_add's multi-launch form, 10 single-launch fwd with the pre-addition fused in, 11-15 the channels-first
+ * kernels (fwd statistics, fwd apply, bwd reduce, bwd dx, dgamma / dbeta).
  */
-#define GNNHWC_NUM_KERNEL_KINDS 11
+#define GNNHWC_NUM_KERNEL_KINDS 16
 int gnnhwc_profile_enable(int on);
 int gnnhwc_profile_collect(int64_t *launches /* [GNNHWC_NUM_KERNEL_KINDS] */,
                            double *total_ms /* [GNNHWC_NUM_KERNEL_KINDS] */);

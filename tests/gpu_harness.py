@@ -98,3 +98,41 @@ def err(a, truth):
 
 def as_np64(t):
     return t.detach().to("cpu", torch.float64).numpy()
+
+
+def cabi_fwd_nchw(x_ncr, w, b, G, eps, act, y=None):
+    """gnnhwc_fwd_nchw on (N, C, R) contiguous device tensors.  Returns y, mean, rstd."""
+    N, C, R = x_ncr.shape
+    dt = DT_CODE[x_ncr.dtype]
+    sdtype = torch.float32 if x_ncr.dtype in (torch.float16, torch.bfloat16) else x_ncr.dtype
+    pdt = DT_CODE[w.dtype] if w is not None else dt
+    y = torch.empty_like(x_ncr) if y is None else y
+    mean = torch.empty((N, G), dtype=sdtype, device=x_ncr.device)
+    rstd = torch.empty((N, G), dtype=sdtype, device=x_ncr.device)
+    lib = _cabi.lib
+    nbytes = lib.gnnhwc_nchw_workspace_bytes(N, C, R, G, dt, 0)
+    assert nbytes > 0, _cabi.last_error()
+    ws = torch.empty((nbytes,), dtype=torch.uint8, device=x_ncr.device)
+    rc = lib.gnnhwc_fwd_nchw(_ptr(x_ncr), _ptr(w), _ptr(b), _ptr(y), _ptr(mean), _ptr(rstd), N, C, R, G, float(eps), int(act),
+                             dt, pdt, DT_CODE[sdtype], _ptr(ws), ws.numel(), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    _cabi.check(rc, "gnnhwc_fwd_nchw")
+    return y, mean, rstd
+
+
+def cabi_bwd_nchw(dy_ncr, x_ncr, w, b, mean, rstd, G, act, want_dw=True, want_db=True):
+    N, C, R = x_ncr.shape
+    dt = DT_CODE[x_ncr.dtype]
+    pdtype = w.dtype if w is not None else x_ncr.dtype
+    dx = torch.empty_like(x_ncr)
+    dw = torch.empty((C,), dtype=pdtype, device=x_ncr.device) if want_dw else None
+    db = torch.empty((C,), dtype=pdtype, device=x_ncr.device) if want_db else None
+    lib = _cabi.lib
+    nbytes = lib.gnnhwc_nchw_workspace_bytes(N, C, R, G, dt, 1)
+    assert nbytes > 0, _cabi.last_error()
+    ws = torch.empty((nbytes,), dtype=torch.uint8, device=x_ncr.device)
+    rc = lib.gnnhwc_bwd_nchw(_ptr(dy_ncr), _ptr(x_ncr), _ptr(w), _ptr(b), _ptr(mean), _ptr(rstd), _ptr(dx), _ptr(dw), _ptr(db),
+                             N, C, R, G, int(act), dt, DT_CODE[pdtype], DT_CODE[mean.dtype], _ptr(ws), ws.numel(),
+                             ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    _cabi.check(rc, "gnnhwc_bwd_nchw")
+    return dx, dw, db
+

@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     assert {"gnnhwc_fwd", "gnnhwc_fwd_add", "gnnhwc_bwd", "gnnhwc_fwd_workspace_bytes", "gnnhwc_bwd_workspace_bytes", "gnnhwc_last_error",
             "gnnhwc_version", "gnnhwc_profile_enable", "gnnhwc_profile_collect", "gnnhwc_kernel_kind_name",
             "gnnhwc_debug_read_trace", "gnnhwc_set_resident", "gnnhwc_debug_copy", "gnnhwc_debug_set_spin_limit",
-            "gnnhwc_debug_plan"} <= set(names)
+            "gnnhwc_debug_plan", "gnnhwc_fwd_nchw", "gnnhwc_bwd_nchw", "gnnhwc_nchw_workspace_bytes"} <= set(names)
     lib = ctypes.CDLL(_cabi.LIB_PATH)
     for n in names:
         assert hasattr(lib, n), n
@@ -112,8 +112,9 @@ def test_ops_are_registered_and_reject_host_tensors():
 
 
 @pytest.mark.parametrize("act", ["identity", "relu", "silu", "gelu", "gelu_tanh"])
-def test_channels_first_input_takes_the_torch_fallback(act):
-    """custom_gn.py:75-79: NCHW input never reaches the kernels, so this path runs on the CPU."""
+def test_channels_first_host_input_takes_the_torch_expression(act):
+    """custom_gn.py:75-79: in the reference channels-first input never reaches a kernel, so that path also serves
+    host tensors; here device tensors get the channels-first kernels and host tensors keep the torch expression."""
     from oracle import gn_oracle as orc
 
     torch.manual_seed(1)
