@@ -238,3 +238,15 @@ def test_tiling_invariants_over_many_shapes():
     out = (ctypes.c_int64 * 12)()
     assert _cabi.lib.gnnhwc_debug_plan(1, 16, 12, 4, 3, 1, 0, out) == -1 and "vector width" in _cabi.last_error()
 
+
+
+def test_channels_first_operators_on_meta_tensors():
+    """gnop::fwd_nchw / gnop::bwd_nchw: contiguous outputs of x's shape, statistics in float32 for 16-bit data."""
+    N, C, R, G = 2, 12, 30, 3
+    X = torch.empty((N, C, R), dtype=torch.float16, device="meta")
+    w = torch.empty((C,), dtype=torch.float32, device="meta")
+    Y, mean, rstd = torch.ops.gnop.fwd_nchw(X, w, w, G, 1e-5, 4)
+    assert Y.shape == X.shape and Y.is_contiguous() and Y.dtype == torch.float16
+    assert mean.shape == (N, G) and mean.dtype == torch.float32 and rstd.shape == (N, G)
+    dX, dw, db = torch.ops.gnop.bwd_nchw(X, X, w, w, mean, rstd, G, 4)
+    assert dX.shape == X.shape and dw.shape == (C,) and dw.dtype == torch.float32 and db.dtype == torch.float32
