@@ -706,7 +706,7 @@ const char *gnnhwc_kernel_kind_name(int kind) {
   static const char *names[GNNHWC_NUM_KERNEL_KINDS] = {"fwd_stats", "fwd_stats_compact", "fwd_apply", "bwd_reduce",
                                                        "bwd_compact", "bwd_dx", "fused_fwd", "fused_bwd", "copy",
                                                        "fwd_add", "fused_fwd_add",
-                                                       "nchw_stats", "nchw_apply", "nchw_bwd_reduce", "nchw_bwd_dx", "nchw_dwdb"};
+                                                       "nchw_stats", "nchw_apply", "nchw_bwd_reduce", "nchw_bwd_dx"};
   return (kind >= 0 && kind < GNNHWC_NUM_KERNEL_KINDS) ? names[kind] : "";
 }
 

@@ -21,11 +21,10 @@ enum KernelKind {
   kKindCopy = 8,
   kKindAdd = 9,        // elementwise pre-addition of the multi-launch fused-addition forward
   kKindFusedFwdAdd = 10,  // single-launch forward with the pre-addition fused in
-  kKindNchwStats = 11,    // channels-first layout: forward statistics, forward apply, backward reduce, backward dx,
-  kKindNchwApply = 12,    // dgamma / dbeta
+  kKindNchwStats = 11,    // channels-first layout: forward statistics, forward apply, backward reduce,
+  kKindNchwApply = 12,    // backward dx (+ dgamma / dbeta)
   kKindNchwBwdReduce = 13,
   kKindNchwBwdDx = 14,
-  kKindNchwDwDb = 15,
   kNumKinds = 9
 };
 

@@ -2,7 +2,7 @@
 //
 // The reference has no kernel for this layout: GN_NHWC.forward hands channels-first input to torch's GroupNorm
 // and applies the activation in a second pass (src/gnnhwc/custom_gn.py:75-79).  Here the same result comes from
-// two launches forward (x is read twice, y written once) and three backward, with the activation fused.
+// two launches forward (x is read twice, y written once) and two backward, with the activation fused.
 //
 // In this layout a (sample, group) slab is D * R contiguous elements and a channel is a contiguous row of R, so
 // the unit of work is one wavefront on one chunk of one row: its 64 lanes read consecutive 16-byte vectors, every
@@ -226,7 +226,8 @@ __global__ __launch_bounds__(kBlock) void nchw_bwd_reduce_kernel(const T *__rest
 template <typename T, typename PT, int VEC, int ACT>
 __global__ __launch_bounds__(kBlock) void nchw_bwd_dx_kernel(const T *__restrict__ x, const T *__restrict__ dy, T *__restrict__ dx,
                                                              const void *mean, const void *rstd, int sdtype, const void *w,
-                                                             const void *b, const acc_t<T> *__restrict__ part, NchwGeo q) {
+                                                             const void *b, const acc_t<T> *__restrict__ part, void *dw, void *db,
+                                                             NchwGeo q) {
   using A = acc_t<T>;
   using LV = LaneVec<T, VEC>;
   NchwPos p;
@@ -244,6 +245,28 @@ __global__ __launch_bounds__(kBlock) void nchw_bwd_dx_kernel(const T *__restrict
   const A beta = b ? load_param<PT, A>(b, p.c) : (A)0;
   const A mu = load_scalar<A>(mean, p.n * q.G + p.g, sdtype);
   const A rs = load_scalar<A>(rstd, p.n * q.G + p.g, sdtype);
+  // dgamma_c = sum_n (S1 - mean S2) rstd and dbeta_c = sum_n S2 (compute_dweight_dbias, gn_kernel.cu:695-728) over
+  // the N * chunks partials of channel c: the wavefront on the channel's first chunk in the first sample does it
+  if (p.n == 0 && p.k == 0 && (dw || db)) {
+    const int64_t plane = q.rows * q.chunks;
+    A t1 = (A)0, t2 = (A)0;
+    const int64_t entries = q.N * q.chunks;
+    for (int64_t i = p.lane; i < entries; i += 64) {
+      const int64_t nn = i / q.chunks;
+      const int kk = (int)(i - nn * q.chunks);
+      const int64_t slot = (nn * q.C + p.c) * q.chunks + kk;
+      const A s1 = part[slot], s2 = part[plane + slot];
+      const A m = load_scalar<A>(mean, nn * q.G + p.g, sdtype);
+      const A r = load_scalar<A>(rstd, nn * q.G + p.g, sdtype);
+      t1 += (s1 - m * s2) * r;
+      t2 += s2;
+    }
+    segment_sum2(t1, t2, 64);
+    if (p.lane == 0) {
+      if (dw) store_param<PT, A>(dw, p.c, t1);
+      if (db) store_param<PT, A>(db, p.c, t2);
+    }
+  }
   // group sums from the slab's D * chunks partials
   A ta = (A)0, tb = (A)0;
   {
@@ -277,37 +300,6 @@ __global__ __launch_bounds__(kBlock) void nchw_bwd_dx_kernel(const T *__restrict
       }
       store_streaming<LV>(out + e, LV::pack(vd));
     }
-  }
-}
-
-// ---------------------------------------------------------------------------------------------
-// Backward pass 3: one wavefront per channel, dgamma_c = sum_n (S1 - mean S2) rstd, dbeta_c = sum_n S2
-// (compute_dweight_dbias, gn_kernel.cu:695-728) over the N * chunks partials of the channel.
-// ---------------------------------------------------------------------------------------------
-template <typename A, typename PT>
-__global__ __launch_bounds__(kBlock) void nchw_dwdb_kernel(const A *__restrict__ part, const void *mean, const void *rstd,
-                                                           int sdtype, void *dw, void *db, NchwGeo q) {
-  const int64_t c = (int64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
-  if (c >= q.C) return;
-  const int lane = threadIdx.x & 63;
-  const int g = (int)(c / q.D);
-  const int64_t plane = q.rows * q.chunks;
-  A t1 = (A)0, t2 = (A)0;
-  const int64_t entries = q.N * q.chunks;
-  for (int64_t i = lane; i < entries; i += 64) {
-    const int64_t n = i / q.chunks;
-    const int k = (int)(i - n * q.chunks);
-    const int64_t slot = (n * q.C + c) * q.chunks + k;
-    const A s1 = part[slot], s2 = part[plane + slot];
-    const A mu = load_scalar<A>(mean, n * q.G + g, sdtype);
-    const A rs = load_scalar<A>(rstd, n * q.G + g, sdtype);
-    t1 += (s1 - mu * s2) * rs;
-    t2 += s2;
-  }
-  segment_sum2(t1, t2, 64);
-  if (lane == 0) {
-    if (dw) store_param<PT, A>(dw, c, t1);
-    if (db) store_param<PT, A>(db, c, t2);
   }
 }
 

@@ -59,10 +59,7 @@ template <typename PT, int VEC, int ACT> void bwd_launch(const NchwArgs &a, cons
   launch(kKindNchwBwdReduce, (nchw_bwd_reduce_kernel<elem_t, PT, VEC, ACT>), dim3(grid), dim3(kBlock), a.stream,
          (const elem_t *)a.x, (const elem_t *)a.dy, a.mean, a.rstd, a.sdtype, a.w, a.b, part, q);
   launch(kKindNchwBwdDx, (nchw_bwd_dx_kernel<elem_t, PT, VEC, ACT>), dim3(grid), dim3(kBlock), a.stream, (const elem_t *)a.x,
-         (const elem_t *)a.dy, (elem_t *)a.dx, a.mean, a.rstd, a.sdtype, a.w, a.b, (const A *)part, q);
-  if (a.dw || a.db)
-    launch(kKindNchwDwDb, (nchw_dwdb_kernel<A, PT>), dim3(wave_grid(q.C)), dim3(kBlock), a.stream, (const A *)part, a.mean, a.rstd,
-           a.sdtype, a.dw, a.db, q);
+         (const elem_t *)a.dy, (elem_t *)a.dx, a.mean, a.rstd, a.sdtype, a.w, a.b, (const A *)part, a.dw, a.db, q);
 }
 template <typename PT, int VEC> void dispatch_act(const NchwArgs &a, const NchwGeo &q) {
   switch (a.act) {

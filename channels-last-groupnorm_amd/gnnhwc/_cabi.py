@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(_CSRC, "libgnnhwc_hip.so")
 
 # dtype / activation codes of include/gnnhwc.h
 F32, F64, F16, BF16 = 0, 1, 2, 3
-NUM_KERNEL_KINDS = 16
+NUM_KERNEL_KINDS = 15
 
 SYMBOLS = (
     "gnnhwc_version",

@@ -133,7 +133,7 @@ int gnnhwc_bwd(const void *dy, const void *x, const void *weight, const void *bi
  * Channels-first layout: x, y, dy, dx are (N, C, R) contiguous, R fastest.  The reference has no kernel for it:
  * GN_NHWC.forward hands such input to torch's GroupNorm and applies the activation in a second pass
  * (custom_gn.py:75-79); these entry points give the same results with the activation fused (forward: two launches,
- * x read twice; backward: three).  Arguments, dtypes, NULL conventions and errors are those of gnnhwc_fwd /
+ * x read twice; backward: two, x and dy read twice).  Arguments, dtypes, NULL conventions and errors are those of gnnhwc_fwd /
  * gnnhwc_bwd, except that C comes before R; y may alias x.  Workspace: gnnhwc_nchw_workspace_bytes.
  */
 size_t gnnhwc_nchw_workspace_bytes(int64_t N, int64_t C, int64_t R, int64_t G, int dtype, int backward);
@@ -172,10 +172,10 @@ int gnnhwc_set_resident(int on);
  * the last collect, then clears the record.  Kinds: 0 fwd statistics, 1 fwd statistics compaction
  * (many row tiles only), 2 fwd apply, 3 bwd reduce, 4 bwd compaction (many row tiles only), 5 bwd dx,
  * 6 single-launch fwd, 7 single-launch bwd, 8 the plain copy of gnnhwc_debug_copy, 9 the elementwise pre-addition
- * of gnnhwc_fwd_add's multi-launch form, 10 single-launch fwd with the pre-addition fused in, 11-15 the channels-first
- * kernels (fwd statistics, fwd apply, bwd reduce, bwd dx, dgamma / dbeta).
+ * of gnnhwc_fwd_add's multi-launch form, 10 single-launch fwd with the pre-addition fused in, 11-14 the channels-first
+ * kernels (fwd statistics, fwd apply, bwd reduce, bwd dx with dgamma / dbeta).
  */
-#define GNNHWC_NUM_KERNEL_KINDS 16
+#define GNNHWC_NUM_KERNEL_KINDS 15
 int gnnhwc_profile_enable(int on);
 int gnnhwc_profile_collect(int64_t *launches /* [GNNHWC_NUM_KERNEL_KINDS] */,
                            double *total_ms /* [GNNHWC_NUM_KERNEL_KINDS] */);
