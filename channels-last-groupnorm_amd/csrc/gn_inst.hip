@@ -187,9 +187,9 @@ template <typename PT, int ACT, int NV, int ADD> bool try_resident_fwd_nv(const 
   return true;
 }
 template <typename PT, int ACT, int ADD> bool try_resident_fwd_add(const FwdArgs &a) {
-  // with a residual the launch holds two tensors, as the backward does, and the alternative is three launches:
-  // the backward's rule for cutting the batch into several single-launch kernels applies
-  const int wb = worthwhile_batches(a.plan, ADD == kAddResidual);
+  // never cut into several launches: with a residual the alternative (an elementwise sum, then the plain forward)
+  // measured faster than two single-launch kernels
+  const int wb = worthwhile_batches(a.plan, false);
   const int most = a.plan.N < wb ? (int)a.plan.N : wb;
   for (int b = 1; b <= most; ++b)
     if (try_resident_fwd_nv<PT, ACT, 4, ADD>(a, b) || try_resident_fwd_nv<PT, ACT, 8, ADD>(a, b) ||
@@ -300,8 +300,16 @@ template <int VEC> hipError_t fwd_impl(const FwdArgs &a) {
     // normalise it from there (in place when it sits in y)
     const Plan &p = a.plan;
     elem_t *dst = (elem_t *)(a.add.sum_out ? a.add.sum_out : a.y);
-    launch(kKindAdd, (add_kernel<elem_t, VEC>), tile_grid(p, 0), dim3(kBlock), a.stream, (const elem_t *)a.x, a.add, dst,
-           (const void *)a.ws, p);
+    if (a.add.residual && !a.add.channel_bias) {
+      const int64_t nvec = p.N * p.R * p.C / VEC;
+      const int64_t want = (nvec + 4 * kBlock - 1) / (4 * kBlock);
+      const unsigned grid = (unsigned)(want < 8 * kNumCU ? (want > 0 ? want : 1) : 8 * kNumCU);
+      launch(kKindAdd, (add_flat_kernel<elem_t, VEC>), dim3(grid), dim3(kBlock), a.stream, (const elem_t *)a.x,
+             (const elem_t *)a.add.residual, dst, nvec);
+    } else {
+      launch(kKindAdd, (add_kernel<elem_t, VEC>), tile_grid(p, 0), dim3(kBlock), a.stream, (const elem_t *)a.x, a.add, dst,
+             (const void *)a.ws, p);
+    }
     FwdArgs plain = a;
     plain.x = dst;
     plain.add = AddArgs{nullptr, nullptr, a.add.channel_bias_dtype, nullptr};

@@ -454,6 +454,38 @@ __global__ __launch_bounds__(kBlock) void add_kernel(const T *__restrict__ x, Ad
   }
 }
 
+// The same without a channel addend: dst = x + residual is a flat elementwise sum, four lane vectors per thread and
+// step (nvec = number of lane vectors of the tensor).
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlock) void add_flat_kernel(const T *__restrict__ x, const T *residual, T *dst, int64_t nvec) {
+  using A = acc_t<T>;
+  using LV = LaneVec<T, VEC>;
+  constexpr int U = 4;
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  for (int64_t i0 = (int64_t)blockIdx.x * kBlock + threadIdx.x; i0 < nvec; i0 += U * stride) {
+    typename LV::raw_t bx[U], br[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t i = i0 + u * stride;
+      const int64_t e = (i < nvec ? i : i0) * VEC;
+      bx[u] = LV::load(x + e);
+      br[u] = LV::load(residual + e);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t i = i0 + u * stride;
+      if (i < nvec) {
+        A vx[VEC], vr[VEC];
+        LV::unpack(bx[u], vx);
+        LV::unpack(br[u], vr);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) vx[j] += vr[j];
+        LV::store(dst + i * VEC, LV::pack(vx));
+      }
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // Forward pass 1: per-tile (count, mean, M2) of every group the tile touches.
 // Does the work of compute_stats_pt1 (src/gnnhwc/csrc/gn_kernel.cu:132-224).
