@@ -148,3 +148,69 @@ def test_random_medium_shapes(family, N, R, C, G, act, dtype, device):
         mask = (z.abs() > RELU_BAND).cpu().numpy()
     for name, ours in (("y", y), ("dx", dx), ("dw", dw), ("db", db)):
         _check(name, ours, as_np64(truth[name]), own and as_np64(own[name]), dtype, mask if name == "dx" else None)
+
+
+def _small_shapes(count, seed):
+    """Seeded sample of small problems with many samples and few channels / rows (where the per-channel reductions
+    over samples and tiles do most of their work): N up to 400, C up to 96, R up to 300."""
+    rng = np.random.RandomState(seed)
+    out = []
+    while len(out) < count:
+        G = int(rng.choice([1, 2, 3, 4, 8, 16]))
+        D = int(rng.choice([1, 2, 3, 4, 6, 8]))
+        C = G * D
+        N = int(rng.choice([1, 2, 7, 33, 65, 129, 200, 400]))
+        R = int(rng.choice([1, 2, 6, 17, 64, 100, 289, 300]))
+        if N * R * C > 2_000_000 or N * R * C < 8:
+            continue
+        out.append((N, R, C, G, ["identity", "relu", "silu", "gelu", "gelu_tanh"][len(out) % 5],
+                    [torch.float32, torch.bfloat16, torch.float64, torch.float16][len(out) % 4]))
+    return out
+
+
+@pytest.mark.parametrize("N,R,C,G,act,dtype", _small_shapes(40, 77))
+def test_random_small_shapes_all_layouts(family, N, R, C, G, act, dtype, device):
+    """Channels-last (both kernel families) and channels-first entry points against the CPU oracle on the same
+    values.  16-bit types are compared with torch's own CPU result in that type, as for the configurations."""
+    from tests.gpu_harness import cabi_bwd_nchw, cabi_fwd_nchw
+
+    print("small", family, N, R, C, G, act, dtype, flush=True)
+    gen = torch.Generator().manual_seed(N * 7919 + R * 31 + C)
+    x = (torch.randn((N, R, C), generator=gen) * 1.3 + torch.randn((C,), generator=gen)).to(dtype)
+    dy = torch.randn((N, R, C), generator=gen).to(dtype)
+    w = (torch.rand((C,), generator=gen) + 0.5).to(dtype)
+    b = (0.1 * torch.randn((C,), generator=gen)).to(dtype)
+    code = orc.ACT_CODES[act]
+    truth = orc.fwd_bwd(as_np64(x), as_np64(w), as_np64(b), as_np64(dy), G, EPS, code)
+    own = None
+    if dtype in (torch.float16, torch.bfloat16):
+        xs = x.permute(0, 2, 1).contiguous().requires_grad_()  # torch's CPU GroupNorm in the same type
+        ws, bs = w.clone().requires_grad_(), b.clone().requires_grad_()
+        ys = orc.torch_act(act)(torch.nn.functional.group_norm(xs, G, ws, bs, EPS))
+        gx, gw, gb = torch.autograd.grad(ys, (xs, ws, bs), dy.permute(0, 2, 1))
+        own = {"y": as_np64(ys.detach().permute(0, 2, 1)), "dx": as_np64(gx.permute(0, 2, 1)), "dw": as_np64(gw), "db": as_np64(gb)}
+    mask = None
+    if act == "relu":
+        D = C // G
+        a = np.repeat(truth["rstd"], D, axis=1) * as_np64(w)[None, :]
+        z = as_np64(x) * a[:, None, :] + (as_np64(b)[None, :] - np.repeat(truth["mean"], D, axis=1) * a)[:, None, :]
+        mask = np.abs(z) > RELU_BAND
+    xd, dyd, wd, bd = x.to(device), dy.to(device), w.to(device), b.to(device)
+    sdt = torch.float64 if dtype == torch.float64 else torch.float32
+    results = {}
+    y, mean, rstd = cabi_fwd(xd, wd, bd, G, EPS, code)
+    dx, dw, db = cabi_bwd(dyd, xd, wd, bd, mean, rstd, G, code)
+    results["channels-last"] = (y, mean, rstd, dx, dw, db)
+    if family == "resident":  # the channels-first kernels have one family: run them once
+        xc, dyc = xd.permute(0, 2, 1).contiguous(), dyd.permute(0, 2, 1).contiguous()
+        yc, meanc, rstdc = cabi_fwd_nchw(xc, wd, bd, G, EPS, code)
+        dxc, dwc, dbc = cabi_bwd_nchw(dyc, xc, wd, bd, meanc, rstdc, G, code)
+        results["channels-first"] = (yc.permute(0, 2, 1), meanc, rstdc, dxc.permute(0, 2, 1), dwc, dbc)
+    torch.cuda.synchronize()
+    for layout, (y, mean, rstd, dx, dw, db) in results.items():
+        _check(layout + " mean", mean, truth["mean"], None, sdt)
+        _check(layout + " rstd", rstd, truth["rstd"], None, sdt)
+        _check(layout + " y", as_np64(y), truth["y"], own and own["y"], dtype)
+        _check(layout + " dx", as_np64(dx), truth["dx"], own and own["dx"], dtype, mask)
+        _check(layout + " dw", dw, truth["dw"], own and own["dw"], dtype)
+        _check(layout + " db", db, truth["db"], own and own["db"], dtype)
