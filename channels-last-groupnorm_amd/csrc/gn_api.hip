@@ -618,6 +618,9 @@ static int nchw_call(NchwArgs &a, int dtype, void *workspace, size_t workspace_b
   if (!workspace || !aligned16(workspace) || workspace_bytes < need)
     return fail(GNNHWC_ERR_WORKSPACE, "%s workspace must be 16-byte aligned and at least %zu bytes (got %p, %zu bytes)", what,
                 need, workspace, workspace_bytes);
+  // the kernels index the elements of one row, and its chunks, with 32-bit integers
+  if (a.R > 0x7fffffffLL - 4096)
+    return fail(GNNHWC_ERR_INVALID_ARGUMENT, "%s: rows of %lld elements are beyond the supported range", what, (long long)a.R);
   const int vec = a.vector ? 16 / (int)elem_size(dtype) : 1;
   const int64_t chunks = (a.R + nchw_chunk_len(vec) - 1) / nchw_chunk_len(vec);
   if ((double)a.N * (double)a.C * (double)chunks / 4.0 > 2.0e9)

@@ -250,3 +250,19 @@ def test_channels_first_operators_on_meta_tensors():
     assert mean.shape == (N, G) and mean.dtype == torch.float32 and rstd.shape == (N, G)
     dX, dw, db = torch.ops.gnop.bwd_nchw(X, X, w, w, mean, rstd, G, 4)
     assert dX.shape == X.shape and dw.shape == (C,) and dw.dtype == torch.float32 and db.dtype == torch.float32
+
+
+def test_channels_first_argument_checks_need_no_gpu():
+    lib = _cabi.lib
+    assert lib.gnnhwc_nchw_workspace_bytes(2, 8, 100, 2, 3, 0) % 256 == 0
+    assert lib.gnnhwc_nchw_workspace_bytes(2, 8, 100, 3, 3, 0) == 0 and "divisible" in _cabi.last_error()
+    one = ctypes.c_void_p(16)  # never dereferenced: every call below fails validation first
+    rc = lib.gnnhwc_fwd_nchw(one, None, None, one, None, None, 1, 8, 16, 2, 1e-5, 9, 0, 0, 0, one, 1 << 20, None)
+    assert rc == -1 and "activation" in _cabi.last_error()
+    rc = lib.gnnhwc_fwd_nchw(one, None, None, one, None, None, 1, 8, 16, 2, 1e-5, 0, 3, 2, 0, one, 1 << 20, None)
+    assert rc == -1 and "dtype" in _cabi.last_error()
+    rc = lib.gnnhwc_bwd_nchw(None, one, None, None, one, one, one, None, None, 1, 8, 16, 2, 0, 0, 0, 0, one, 1 << 20, None)
+    assert rc == -1 and "must not be null" in _cabi.last_error()
+    rc = lib.gnnhwc_fwd_nchw(one, None, None, one, None, None, 1, 2, 2 ** 31, 1, 1e-5, 0, 0, 0, 0, one, 1 << 40, None)
+    assert rc == -1 and "beyond the supported range" in _cabi.last_error()
+
