@@ -54,6 +54,10 @@ def parse_args():
     ap.add_argument("--nchw", action="store_true",
                     help="also time the channels-first entry points on the same shapes against torch's GroupNorm + activation "
                          "on channels-first tensors (reported under 'channels_first')")
+    ap.add_argument("--timeline", action="store_true",
+                    help="no headline: print the in-kernel timeline of the single-launch kernels (wall-clock stamps every workgroup "
+                         "takes at its phase boundaries; min / median / max over the workgroups of one launch) for each shape of "
+                         "the workload (default here: c3a c3b c3c c4a), forward and backward")
     ap.add_argument("--counter-workload", action="store_true",
                     help="no timing: one 256 MiB plain copy (calibration) and a few fwd+bwd calls per shape, for a rocprofv3 --pmc run")
     return ap.parse_args()
@@ -64,8 +68,8 @@ class Problem:
 
     def __init__(self, cfg, device, nsets=1):
         import torch
-        from tests import configs
-        from tests.gpu_harness import nrc_view
+        import workloads as configs
+        from workloads import nrc_view
 
         self.cfg = cfg
         self.S = configs.tensor_bytes(cfg)
@@ -88,7 +92,7 @@ class Problem:
         self.dw = torch.empty((self.C,), dtype=self.w.dtype, device=device)
         self.db = torch.empty((self.C,), dtype=self.w.dtype, device=device)
         from gnnhwc import _cabi
-        from tests.gpu_harness import DT_CODE
+        from workloads import DT_CODE
 
         self.lib = _cabi.lib
         self.dt = DT_CODE[x.dtype]
@@ -286,11 +290,80 @@ def counter_workload(probs, device):
     print(json.dumps({"counter_workload": [p.cfg.name for p in probs], "copy_bytes": n}))
 
 
+FWD_STAMPS = ((0, "workgroup starts"), (1, "tile moments in registers (all rows arrived)"), (2, "tile reduced, records published"),
+              (3, "other tiles' records seen, statistics merged"), (4, "rows normalised and stored"))
+BWD_STAMPS = ((0, "workgroup starts"), (1, "mean / rstd staged"), (6, "tile sums in registers (all rows arrived)"),
+              (2, "tile reduced, records published"), (3, "other tiles' records seen, coefficients merged"), (4, "dx stored"),
+              (5, "dgamma / dbeta written (workgroups of sample 0)"))
+
+
+def timeline(names, device, reps=5):
+    """In-kernel timeline of the single-launch kernels.  Thread 0 of every workgroup stamps a 100 MHz wall clock at its
+    phase boundaries (GNNHWC_TRACE=2: the stamps do not wait for outstanding memory operations, so the kernel overlaps
+    as it does untraced); the stamps of the most recent launch are read back and reported relative to the earliest
+    workgroup start of that launch, in microseconds, as min / median / max over its workgroups.  The event-timed
+    duration of the same launch (begin to end of the dispatch) is printed beside it."""
+    import numpy as np
+    import torch
+    from gnnhwc import _cabi
+    import workloads as configs
+
+    stream = torch.cuda.current_stream().cuda_stream
+    words = np.zeros((1024, 8), dtype=np.uint64)
+    print("# in-kernel timeline, microseconds after the first workgroup of the launch started: min / median / max over workgroups")
+    for name in names:
+        p = Problem(configs.CONFIGS[name], device)
+        for which, stamps in (("fwd", FWD_STAMPS), ("bwd", BWD_STAMPS)):
+            if which == "bwd" and not p.bwd:
+                continue
+            for _ in range(3):
+                p.step(0, stream)
+            torch.cuda.synchronize()
+            time.sleep(0.002)  # stamps of earlier launches end up far behind those of the launches below
+            _cabi.profile_enable(True)
+            for _ in range(20):
+                p.step(0, stream, which)
+            _cabi.profile_enable(False)
+            res = {k: v for k, v in _cabi.profile_collect().items() if v[0]}
+            kinds = ", ".join("%s %.2f us x %d per call" % (k, ms / n * 1e3, n // 20) for k, (n, ms) in res.items())
+            if not any(k.startswith("fused") for k in res):
+                print("%s %s: multi-launch kernels (no in-kernel timeline); event-timed: %s" % (name, which, kinds))
+                continue
+            torch.cuda.synchronize()
+            time.sleep(0.002)
+            rows = []
+            for _ in range(reps):
+                p.step(0, stream, "both" if which == "bwd" else "fwd")  # a backward is measured behind its own forward, as in the sweep
+                torch.cuda.synchronize()
+                _cabi.check(_cabi.lib.gnnhwc_debug_read_trace(words.ctypes.data, words.size), "gnnhwc_debug_read_trace")
+                t = words.astype(np.int64)
+                live = t[:, 0] >= t[:, 0].max() - 5000  # within 50 us of the latest start: this launch
+                t = t[live]
+                rel = (t - t[:, 0].min()) / 100.0
+                taken = {}
+                for pt, _ in stamps:  # a stamp older than the launch was not taken by this launch (stamp 5: sample 0 only)
+                    v = rel[:, pt][t[:, pt] >= t[:, 0].min()]
+                    if v.size:
+                        taken[pt] = (float(v.min()), float(np.median(v)), float(v.max()))
+                rows.append((int(live.sum()), taken))
+                time.sleep(0.002)
+            nwg = rows[-1][0]
+            print("%s %s: %d workgroups in the traced launch; event-timed: %s" % (name, which, nwg, kinds))
+            for pt, label in stamps:
+                vals = [r[1][pt] for r in rows if pt in r[1]]
+                if not vals:
+                    continue
+                med = [statistics.median(v[i] for v in vals) for i in range(3)]
+                print("    %-58s %7.2f / %7.2f / %7.2f" % (label, med[0], med[1], med[2]))
+        del p
+        torch.cuda.empty_cache()
+
+
 def cpu_baseline(cfg_names, seconds):
     """torch's CPU GroupNorm + activation + autograd on the host cores, same seeded tensors and dtype."""
     import torch
     from oracle import gn_oracle as orc  # the checker's torch_reference: the CPU baseline leg
-    from tests import configs
+    import workloads as configs
 
     per = {}
     total_bytes, total_time = 0.0, 0.0
@@ -353,7 +426,7 @@ def fused_add_table(names, device, steps, warmup):
     4 S algorithmic bytes) against the unfused sequence a caller of the plain forward runs (torch.add into a sum
     buffer, then gnnhwc_fwd on it: 3 S + 2 S), and the channel-bias-only form (2 S) against its unfused sequence."""
     import torch
-    from tests import configs
+    import workloads as configs
 
     out = {}
     for n in names:
@@ -415,8 +488,8 @@ def nchw_table(names, device, steps, warmup):
     activation, and their autograd backward."""
     import torch
     import torch.nn.functional as F
-    from tests import configs
-    from tests.gpu_harness import DT_CODE
+    import workloads as configs
+    from workloads import DT_CODE
 
     acts = {"identity": lambda t: t, "relu": F.relu, "silu": F.silu, "gelu": F.gelu,
             "gelu_tanh": lambda t: F.gelu(t, approximate="tanh")}
@@ -485,8 +558,10 @@ def main():
         print("bench.py: this build measures one GPU only (GroupNorm statistics are per sample; nothing is exchanged "
               "between GPUs). Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
+    if args.timeline:
+        os.environ["GNNHWC_TRACE"] = "2"  # read by the library at its first single-launch call
     import torch
-    from tests import configs
+    import workloads as configs
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
@@ -494,6 +569,10 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
     use_graph = args.graph
+    if args.timeline:
+        timeline(["c3a", "c3b", "c3c", "c4a"] if args.workload == "sd_unet" else
+                 list(configs.ALL_NAMES) if args.workload == "all" else [args.workload], device)
+        return
 
     if args.workload == "sd_unet":
         head_names = list(configs.SD_UNET_SWEEP)

@@ -380,7 +380,8 @@ int resident_min_rows() {
   static const int v = env_int("GNNHWC_RESIDENT_MIN_ROWS", 0);
   return v;
 }
-std::atomic<int> g_spin_limit{1 << 22};
+constexpr int kDefaultSpinLimit = 1 << 20;  // polls per wait; a poll is a device-scope round trip, about a microsecond
+std::atomic<int> g_spin_limit{kDefaultSpinLimit};
 int resident_spin_limit() { return g_spin_limit.load(std::memory_order_relaxed); }
 
 std::atomic<int> g_resident{-1};  // -1: follow the environment
@@ -569,6 +570,8 @@ int gnnhwc_profile_collect(int64_t *launches, double *total_ms) {
   return rc;
 }
 
+int gnnhwc_resident_status(void) { return check_resident_health(); }
+
 int gnnhwc_set_resident(int on) {
   const int before = resident_enabled() ? 1 : 0;
   g_resident.store(on ? 1 : 0, std::memory_order_relaxed);
@@ -576,7 +579,7 @@ int gnnhwc_set_resident(int on) {
 }
 
 int gnnhwc_debug_set_spin_limit(int polls) {
-  if (polls < 0) polls = 1 << 22;
+  if (polls < 0 && polls != -2) polls = kDefaultSpinLimit;  // -2: every wait gives up at its first poll, ready or not
   return g_spin_limit.exchange(polls, std::memory_order_relaxed);
 }
 
@@ -614,6 +617,8 @@ size_t gnnhwc_nchw_workspace_bytes(int64_t N, int64_t C, int64_t R, int64_t G, i
   return align_up(nchw_workspace_elems(N, C, R, 1, backward != 0) * acc_size(dtype), 256);
 }
 static int nchw_call(NchwArgs &a, int dtype, void *workspace, size_t workspace_bytes, const char *what) {
+  const int health = check_resident_health();  // an earlier single-launch call of the process may have failed
+  if (health != GNNHWC_OK) return health;
   const size_t need = gnnhwc_nchw_workspace_bytes(a.N, a.C, a.R, a.G, dtype, a.backward ? 1 : 0);
   if (!workspace || !aligned16(workspace) || workspace_bytes < need)
     return fail(GNNHWC_ERR_WORKSPACE, "%s workspace must be 16-byte aligned and at least %zu bytes (got %p, %zu bytes)", what,

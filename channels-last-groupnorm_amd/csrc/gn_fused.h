@@ -14,25 +14,29 @@
 // make ordinary stores visible across them (L2 write-back / invalidate) cost tens of microseconds when
 // every workgroup issues them.  So everything that crosses workgroups is written with device-scope
 // (write-through) stores and read with device-scope (cache-bypassing) loads, and no fence is used.
-//  * Per-group tile results travel as 16-byte records {value0, value1, epoch (64 bit)} written by a
-//    single 128-bit store and read by a single 128-bit load: a consumer that sees this call's epoch in a
-//    record has the values that were stored with it.  The epoch is a fresh 64-bit value per call, so
-//    the workspace never needs clearing.  One memory round trip carries both "ready" and the data.
-//  * Per-channel sums for dgamma / dbeta use a flag per workgroup: every wave waits for the
-//    acknowledgement of its device-scope stores (s_waitcnt 0), the workgroup barriers, one thread
-//    stores the flag; the consumer loads the data only after it has seen the flag.
-// Polling is bounded by kMaxSpins; a timeout only records the epoch in a status word, so the grid
-// always drains.  Only fp32-accumulating element types use these kernels (a record has room for two
-// 32-bit values); float64 data takes the streaming kernels.
+//  * Everything that crosses workgroups travels as a 16-byte record {value0, value1, epoch (64 bit)} written by a
+//    single 128-bit store and read by a single 128-bit load: per (sample, chunk, group, tile) for the group
+//    statistics / group sums, and in the backward per (sample, tile, channel) for the sums that feed dgamma / dbeta.
+//    A consumer that sees this call's epoch in a record takes the values it loaded with it.  The epoch is a fresh
+//    64-bit value per call, so the workspace never needs clearing, there are no flags, and one memory round trip
+//    carries both "ready" and the data.
+//    This relies on an aligned 128-bit device-scope store being observed as a whole by an aligned 128-bit
+//    device-scope load (single-copy atomicity of a 16-byte access inside one 64-byte sector of the memory channel
+//    that owns it).  The instruction set does not promise it in writing; if it did not hold, a consumer could pair a
+//    fresh epoch with stale values.  The epoch therefore sits in the LAST two words of the record: a torn access
+//    that delivered the words in address order would show stale epoch words, not stale values.
+// Polling is bounded (SyncArea::max_spins).  A wait that expires records the epoch in a host-visible status word and
+// poisons what depended on it with NaN, and the kernel carries on: the grid always drains.  Only fp32-accumulating
+// element types use these kernels (a record has room for two 32-bit values); float64 data takes the streaming kernels.
 #pragma once
 #include "gn_kernels.h"
 
 namespace gn {
 
-constexpr int kMaxSpins = 1 << 22;  // default bound on the polls of one wait (seconds of polling)
-constexpr int kRecFast = 2;
+constexpr int kRecFast = 2;  // records a lane keeps in registers while polling
+constexpr int kForcedTimeout = -2;  // poll limit that makes every wait give up at once (tests of the failure path)
 constexpr int kTailFast = 2;  // channel records a lane of the dgamma / dbeta stage requests ahead of the dx phase
-constexpr int kMaxResidentBlocksDev = 4 * kNumCU;  // records a lane keeps in registers while polling
+constexpr int kMaxResidentBlocksDev = 4 * kNumCU;
 
 struct SyncArea {
   void *recs;                 // 16-byte records, laid out [N][nchunk][G][tiles]
@@ -114,12 +118,12 @@ __device__ __forceinline__ int record_slot(const PartialGeo &q, int G, int n, in
   return __mul24(__mul24(col, G) + g, q.tiles) + t;
 }
 
-// Collect the records of group g (all tiles of the chunks that hold a piece of it) with L lanes and reduce
-// them with reduce(e0[], e1[], cnt[], n_mine): each lane polls its own records until they carry this call's
-// epoch.  Up to kRecFast records per lane stay in registers (one round trip); more are polled first and
-// then re-read.  Returns through `out` whatever reduce produces from (value0, value1, count) per record.
+// Collect the records of group g (all tiles of the chunks that hold a piece of it) with L lanes: each lane polls its
+// own records until they carry this call's epoch, kRecFast at a time (they stay in registers: the round trip that
+// finds them ready also brings their values), and hands (value0, value1, count) of each to body.  Returns false if
+// a wait expired: the lane's records are then not this call's, and the caller must not produce a plausible result.
 template <typename BODY>
-__device__ __forceinline__ void for_group_records(const SyncArea &s, __amdgpu_buffer_rsrc_t rb, const PartialGeo &q,
+__device__ __forceinline__ bool for_group_records(const SyncArea &s, __amdgpu_buffer_rsrc_t rb, const PartialGeo &q,
                                                   const Plan &p, int64_t n, int g, bool valid, int L, int sl, BODY &&body) {
   int k_lo = 0, nk = 1;
   if (valid) group_chunks(q, p.D, g, k_lo, nk);
@@ -127,6 +131,7 @@ __device__ __forceinline__ void for_group_records(const SyncArea &s, __amdgpu_bu
   const int base = record_slot(q, p.G, (int)n, 0, k_lo, g);
   const int kstride = __mul24(p.G, q.tiles);
   int spins = 0;
+  bool good = true;
   for (int e0 = sl; e0 < P; e0 += kRecFast * L) {
     u32x4 rec[kRecFast];
     bool have[kRecFast];
@@ -146,9 +151,11 @@ __device__ __forceinline__ void for_group_records(const SyncArea &s, __amdgpu_bu
       for (int i = 0; i < kRecFast; ++i) rec[i] = record_load(rb, idx[i]);
 #pragma unroll
       for (int i = 0; i < kRecFast; ++i) ok = ok && (!have[i] || record_ready(rec[i], s.epoch));
+      if (s.max_spins == kForcedTimeout) ok = false;
       if (ok) break;
       if (++spins > s.max_spins) {
         *s.status = s.epoch;
+        good = false;
         break;
       }
       __builtin_amdgcn_s_sleep(2);
@@ -162,7 +169,10 @@ __device__ __forceinline__ void for_group_records(const SyncArea &s, __amdgpu_bu
       }
     }
   }
+  return good;
 }
+// What a result is replaced by when a wait expired: not a number, so that the call's output cannot pass for one.
+__device__ __forceinline__ float poison() { return __builtin_nanf(""); }
 
 // ---------------------------------------------------------------------------------------------
 // Resident forward.  NV = register capacity in rows per lane.  Statistics follow the same definitions
@@ -310,13 +320,14 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
       const int g = l.g_lo + gi;
       // each lane folds its records about the mean of its first one ...
       A nl = (A)0, kl = (A)0, s1 = (A)0, s2 = (A)0;
-      for_group_records(sync, rb, q, p, n, g, valid, L, sl, [&](float mu, float mm, float cnt) {
+      const bool good = for_group_records(sync, rb, q, p, n, g, valid, L, sl, [&](float mu, float mm, float cnt) {
         if (nl == (A)0) kl = mu;
         const A d = mu - kl;
         nl += cnt;
         s1 += cnt * d;
         s2 += mm + cnt * d * d;
       });
+      if (!good) s1 = poison();  // reaches mean and rstd of the group, and through them every y of this tile
       const A inv = nl > (A)0 ? fast_rcp(nl) : (A)0;
       const A mean_l = kl + s1 * inv;
       const A m2_l = s2 - s1 * s1 * inv;
@@ -511,10 +522,11 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
       const bool valid = gi < l.ng;
       const int g = l.g_lo + gi;
       A ta = (A)0, tb = (A)0;
-      for_group_records(sync, rb, q, p, n, g, valid, L, sl, [&](float ra, float rbv, float) {
+      const bool good = for_group_records(sync, rb, q, p, n, g, valid, L, sl, [&](float ra, float rbv, float) {
         ta += ra;
         tb += rbv;
       });
+      if (!good) ta = poison();  // reaches both coefficients of the group, and through them every dx of this tile
       segment_sum2(ta, tb, L);
       if (valid && sl == 0) {
         const A mu = sm_mu[gi];
@@ -588,6 +600,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
   trace_point(sync, 4);
   if (tail) {
     int spins = 0;
+    bool tail_good = true;
     for (int cb = l.tile * cpp; cb < l.wch; cb += p.tiles * cpp) {
       const bool first = cb == l.tile * cpp;
       const int cc = cb + tslot;
@@ -599,9 +612,10 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
       auto add = [&](int e, u32x4 rec, A mu, A rs) {
         const int64_t nn = e / p.tiles;
         const int t = e - (int)nn * p.tiles;
-        while (valid && nn >= n0 && !record_ready(rec, sync.epoch)) {
+        while (valid && nn >= n0 && (!record_ready(rec, sync.epoch) || sync.max_spins == kForcedTimeout)) {
           if (++spins > sync.max_spins) {
             *sync.status = sync.epoch;
+            tail_good = false;
             break;
           }
           __builtin_amdgcn_s_sleep(2);
@@ -627,6 +641,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
             load_scalar<A>(rstd_all, nn * p.G + g, sdtype));
       }
       if (!valid) { t1 = (A)0; t2 = (A)0; }
+      if (!tail_good) { t1 = poison(); t2 = poison(); }  // a wait expired: dgamma / dbeta of these channels say so
       segment_sum2(t1, t2, TL);
       if (valid && tsl == 0) {
         if (dw) store_param<PT, A>(dw, c, t1);

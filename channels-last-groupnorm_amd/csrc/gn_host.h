@@ -5,6 +5,7 @@
 #include <hip/hip_ext.h>
 #include <stddef.h>
 #include <stdint.h>
+#include "../../include/gnnhwc.h"
 #include "gn_plan.h"
 
 namespace gn {
@@ -25,8 +26,9 @@ enum KernelKind {
   kKindNchwApply = 12,    // backward dx (+ dgamma / dbeta)
   kKindNchwBwdReduce = 13,
   kKindNchwBwdDx = 14,
-  kNumKinds = 9
+  kNumKinds = 15
 };
+static_assert(kNumKinds == GNNHWC_NUM_KERNEL_KINDS, "kernel kinds out of step with include/gnnhwc.h");
 
 struct FwdArgs {
   const void *x, *w, *b;

@@ -101,6 +101,7 @@ bool resident_tiling(const Plan &base, int64_t samples, int nv, int slots, Plan 
   return true;
 }
 
+
 struct ResidentWorkspace {
   SyncArea sync;
 };

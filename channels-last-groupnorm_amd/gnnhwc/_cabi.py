@@ -29,6 +29,7 @@ SYMBOLS = (
     "gnnhwc_profile_collect",
     "gnnhwc_kernel_kind_name",
     "gnnhwc_set_resident",
+    "gnnhwc_resident_status",
     "gnnhwc_debug_read_trace",
     "gnnhwc_debug_plan",
 )
@@ -69,6 +70,8 @@ def _load():
     lib.gnnhwc_profile_collect.restype = ci
     lib.gnnhwc_set_resident.argtypes = [ci]
     lib.gnnhwc_set_resident.restype = ci
+    lib.gnnhwc_resident_status.argtypes = []
+    lib.gnnhwc_resident_status.restype = ci
     lib.gnnhwc_debug_read_trace.argtypes = [vp, i64]
     lib.gnnhwc_debug_read_trace.restype = ci
     lib.gnnhwc_debug_set_spin_limit.argtypes = [ci]

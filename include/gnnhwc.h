@@ -15,9 +15,18 @@
  *   weight, bias, dweight, dbias : (C) in `param_dtype`; weight/bias may be NULL (gamma=1, beta=0).
  *   mean, rstd   : (N, G) in `stats_dtype`.
  * All pointers are device pointers on the device that is current for the calling thread.
- * Calls are asynchronous on `stream` and never synchronise; the library is stateless apart from a
- * per-thread error string, so concurrent calls on different streams are safe as long as each call
- * has its own workspace.
+ * Calls are asynchronous on `stream` and never synchronise.  gnnhwc_fwd / gnnhwc_bwd allocate no device memory: the
+ * caller brings the workspace.  Concurrent calls on different streams are safe as long as each call has its own
+ * workspace.
+ *
+ * State the library keeps (none of it affects results): a per-thread error string; and, for the single-launch
+ * kernels (see gnnhwc_set_resident), process-wide: the on / off switch, per device the stream of the last
+ * single-launch call and one event that orders a call on another stream behind it, a 64-byte host-pinned status
+ * word (allocated with hipHostMalloc at the first single-launch call of the process), one 8-byte generation cell per
+ * device inside the library's image (used by launches recorded into HIP graphs), a pool of events while
+ * gnnhwc_profile_enable is on, and a device buffer of 64 KiB when GNNHWC_TRACE is set in the environment.
+ * A caller that must see no allocation at all after start-up either makes one warm-up call per device first or
+ * switches the single-launch kernels off.
  *
  * Every entry point returns GNNHWC_OK (0) or a negative error code; gnnhwc_last_error() describes the
  * most recent failure on the calling thread.  Nothing is launched when an error is returned.
@@ -183,12 +192,22 @@ const char *gnnhwc_kernel_kind_name(int kind);
 
 /*
  * Failure handling of the single-launch kernels (no counterpart in the reference).  Their workgroups wait for
- * each other with a bounded number of polls; if a wait expires (the workgroups were not all resident at once)
- * the kernel still ends normally, its output is invalid, and the NEXT gnnhwc_fwd / gnnhwc_bwd call on any
- * thread returns GNNHWC_ERR_LAUNCH without launching anything and switches the process to the multi-launch
- * kernels.  gnnhwc_debug_set_spin_limit sets the number of polls per wait (negative: the default, 2^22) and
- * returns the previous value; tests use 0 to exercise this path without hanging anything.
+ * each other with a bounded number of polls.  If a wait expires (the workgroups were not all resident at once: another
+ * process or a concurrently replayed graph held part of the device), the kernel still ends normally, and
+ *   - everything that depended on the expired wait is written as NaN: mean / rstd of the group, every y (dx) element
+ *     of the tiles that waited for it, dweight / dbias of the channels concerned.  The output of the failed call
+ *     cannot be mistaken for a result;
+ *   - a host-visible status word is set.  gnnhwc_resident_status() reads and clears it: it returns GNNHWC_OK, or
+ *     GNNHWC_ERR_LAUNCH (with a message) if a single-launch kernel of this process has failed since the last check.
+ *     It does not synchronise: call it once the work in question has completed (after a stream or event
+ *     synchronisation, after a graph replay has finished).  The next gnnhwc_fwd / gnnhwc_bwd / gnnhwc_fwd_nchw /
+ *     gnnhwc_bwd_nchw call on any thread performs the same check, returns that error without launching anything,
+ *     and the process uses the multi-launch kernels from then on.
+ * gnnhwc_debug_set_spin_limit sets the number of polls per wait and returns the previous value: negative restores the
+ * default (2^20, about a second), except -2, which makes every wait give up at its first poll whether or not the
+ * data had arrived; tests use that to exercise this path, every kernel still exits normally.
  */
+int gnnhwc_resident_status(void);
 int gnnhwc_debug_set_spin_limit(int polls);
 
 /*

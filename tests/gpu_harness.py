@@ -7,19 +7,11 @@ import torch
 
 from gnnhwc import _cabi
 
-DT_CODE = {torch.float32: 0, torch.float64: 1, torch.float16: 2, torch.bfloat16: 3}
+from workloads import DT_CODE, nrc_view  # noqa: F401  (re-exported: the tests import them from here)
 
 
 def _ptr(t):
     return ctypes.c_void_p(t.data_ptr()) if t is not None else None
-
-
-def nrc_view(t):
-    """(N, C, *spatial) tensor with channels fastest -> (N, R, C) contiguous tensor (no copy when already laid out so)."""
-    nd = t.dim()
-    u = t.permute(0, *range(2, nd), 1)
-    u = u if u.is_contiguous() else u.contiguous()
-    return u.reshape(u.shape[0], -1, u.shape[-1])
 
 
 def cabi_fwd(x_nrc, w, b, G, eps, act, stats_dtype=None, y=None, ws=None):

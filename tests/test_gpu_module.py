@@ -405,25 +405,35 @@ def test_inference_in_place_without_statistics(family, shape, G, device):
 
 
 def test_single_launch_timeout_is_reported(device):
-    """A single-launch kernel whose workgroups cannot wait for each other (forced here from the host with a poll
-    limit of 0, so every kernel still ends normally) leaves invalid output; the next call must say so, and the
-    calls after it run on the multi-launch kernels with correct results."""
+    """A single-launch kernel whose workgroups cannot wait for each other (forced here from the host with the poll
+    limit -2: every wait gives up at its first poll, ready or not, and every kernel still ends normally) must not leave
+    anything that could pass for a result: mean, rstd, y, dx, dweight and dbias of the failed calls are NaN, the status
+    query and the next call say so, and the calls after that run on the multi-launch kernels with correct results."""
     lib = _cabi.lib
     gen = torch.Generator().manual_seed(11)
-    N, R, C, G = 1, 4096, 1280, 32  # hundreds of workgroups: some poll is bound to come before its record
+    N, R, C, G = 2, 2048, 1280, 32
     x = (torch.randn((N, R, C), generator=gen) * 2 + 1).to(torch.bfloat16).to(device)
+    dy = torch.randn((N, R, C), generator=gen).to(torch.bfloat16).to(device)
     w = (torch.rand(C, generator=gen) + 0.5).to(torch.bfloat16).to(device)
     b = (0.1 * torch.randn(C, generator=gen)).to(torch.bfloat16).to(device)
     truth = orc.fwd_bwd(x.double().cpu().numpy(), w.double().cpu().numpy(), b.double().cpu().numpy(),
-                        np.zeros((N, R, C)), G, 1e-5, 2)
+                        dy.double().cpu().numpy(), G, 1e-5, 2)
     before = _cabi.set_resident(True)
-    prev = lib.gnnhwc_debug_set_spin_limit(0)
+    good_mean = torch.as_tensor(truth["mean"], dtype=torch.float32, device=device)
+    good_rstd = torch.as_tensor(truth["rstd"], dtype=torch.float32, device=device)
+    prev = lib.gnnhwc_debug_set_spin_limit(-2)
     try:
-        cabi_fwd(x, w, b, G, 1e-5, 2)
+        assert lib.gnnhwc_resident_status() == 0
+        y, mean, rstd = cabi_fwd(x, w, b, G, 1e-5, 2)
         torch.cuda.synchronize()
-    finally:
+        assert bool(torch.isnan(mean).all()) and bool(torch.isnan(rstd).all()) and bool(torch.isnan(y.float()).all())
+        assert lib.gnnhwc_resident_status() == -3 and "could not synchronise" in _cabi.last_error()
+        assert lib.gnnhwc_resident_status() == 0  # reading clears it
+        _cabi.set_resident(True)  # (a reported failure switches the process to the multi-launch kernels)
+        dx, dw, db = cabi_bwd(dy, x, w, b, good_mean, good_rstd, G, 2)
+        torch.cuda.synchronize()
+        assert bool(torch.isnan(dx.float()).all()) and bool(torch.isnan(dw.float()).all()) and bool(torch.isnan(db.float()).all())
         lib.gnnhwc_debug_set_spin_limit(prev)
-    try:
         with pytest.raises(RuntimeError, match="could not synchronise"):
             cabi_fwd(x, w, b, G, 1e-5, 2)
         y, mean, rstd = cabi_fwd(x, w, b, G, 1e-5, 2)  # multi-launch kernels from here on
@@ -431,10 +441,15 @@ def test_single_launch_timeout_is_reported(device):
         assert err(mean, truth["mean"]) <= 1e-5 and err(rstd, truth["rstd"]) <= 1e-5
         assert err(y, truth["y"]) <= 2.0 ** -7
         _cabi.set_resident(True)  # an explicit request re-enables the single-launch kernels
-        y2, mean2, _ = cabi_fwd(x, w, b, G, 1e-5, 2)
+        y2, mean2, rstd2 = cabi_fwd(x, w, b, G, 1e-5, 2)
+        dx2, dw2, db2 = cabi_bwd(dy, x, w, b, mean2, rstd2, G, 2)
         torch.cuda.synchronize()
         assert err(mean2, truth["mean"]) <= 1e-5 and err(y2, truth["y"]) <= 2.0 ** -7
+        assert err(dx2, truth["dx"]) <= 2.0 ** -6 and err(dw2, truth["dw"]) <= 2.0 ** -7 and err(db2, truth["db"]) <= 2.0 ** -7
+        assert lib.gnnhwc_resident_status() == 0
     finally:
+        lib.gnnhwc_debug_set_spin_limit(prev)
+        lib.gnnhwc_resident_status()
         _cabi.set_resident(before)
 
 
