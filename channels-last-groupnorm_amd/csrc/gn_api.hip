@@ -159,14 +159,14 @@ bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 size_t acc_size(int dtype) { return dtype == GN_F64 ? 8 : 4; }
 size_t max_size(size_t a, size_t b) { return a > b ? a : b; }
-size_t fwd_ws_bytes(int64_t N, int64_t R, int64_t C, int64_t G, int dtype) {
+size_t fwd_ws_bytes(int64_t N, int64_t R, int64_t C, int64_t G, int dtype, bool streaming_only = false) {
   const int vec = 16 / elem_size(dtype);
   size_t need = fwd_workspace(make_plan(N, R, C, G, 1, 1)).total;
   size_t resident = 0;
   if (C % vec == 0) {
     const size_t v = fwd_workspace(make_plan(N, R, C, G, vec, 1)).total;
     if (v > need) need = v;
-    resident = dtype == GN_F64 ? 0 : resident_fwd_bytes(G);
+    resident = dtype == GN_F64 || streaming_only ? 0 : resident_fwd_bytes(G);
   }
   return max_size(kWorkspaceHeader + need * acc_size(dtype), resident);
 }
@@ -422,6 +422,46 @@ static int check_resident_health() {
               "The multi-launch kernels are used from now on");
 }
 
+// ---- forward that allocates nothing -------------------------------------------------------------------------
+// The scratch memory of the multi-launch forward (per-tile partial statistics) in the library's own device image:
+// every device the library runs on holds its own copy of this array, at its own address, until the process ends.
+// Host code never uses the array's name as an address: static_scratch() asks the runtime for the current device's
+// copy once and hands that pointer on.
+static __device__ __align__(256) unsigned char scratch[GNNHWC_STATIC_SCRATCH_BYTES];
+namespace {
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices];
+bool g_scratch_tried[kMaxDevices];
+// Address of the current device's copy of `scratch` (null, with the error string set, if it cannot be had).
+void *static_scratch() {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();
+    fail(GNNHWC_ERR_LAUNCH, "no current device for the library's scratch memory (%s)", hipGetErrorString(e));
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_tried[dev]) {
+    // looking a symbol up is not a stream operation, but a capture in progress on this thread must not see it as one
+    hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+    const bool swapped = hipThreadExchangeStreamCaptureMode(&mode) == hipSuccess;
+    void *ptr = nullptr;
+    e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+    if (swapped) (void)hipThreadExchangeStreamCaptureMode(&mode);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      fail(GNNHWC_ERR_LAUNCH, "hipGetSymbolAddress for the library's scratch memory failed: %s", hipGetErrorString(e));
+      return nullptr;  // not marked as tried: a later call asks again
+    }
+    g_scratch_ptr[dev] = ptr;
+    g_scratch_tried[dev] = true;
+  }
+  if (!g_scratch_ptr[dev]) fail(GNNHWC_ERR_LAUNCH, "the library's scratch memory has no address on device %d", dev);
+  return g_scratch_ptr[dev];
+}
+}  // namespace
+
 extern "C" {
 
 int gnnhwc_version(void) { return (1 << 16) | 0; }
@@ -441,7 +481,7 @@ size_t gnnhwc_bwd_workspace_bytes(int64_t N, int64_t R, int64_t C, int64_t G, in
 
 static int forward(const void *x, const AddArgs &add, const void *weight, const void *bias, void *y, void *mean, void *rstd,
                    int64_t N, int64_t R, int64_t C, int64_t G, double eps, int act, int dtype, int param_dtype,
-                   int stats_dtype, void *workspace, size_t workspace_bytes, void *stream) {
+                   int stats_dtype, void *workspace, size_t workspace_bytes, void *stream, bool streaming_only = false) {
   int rc = check_shape(N, R, C, G, dtype);
   if (rc != GNNHWC_OK) return rc;
   rc = check_dtypes(dtype, param_dtype, stats_dtype);
@@ -452,13 +492,14 @@ static int forward(const void *x, const AddArgs &add, const void *weight, const 
   rc = check_resident_health();
   if (rc != GNNHWC_OK) return rc;
   if (!x || !y) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "x and y must not be null");
-  const size_t need = gnnhwc_fwd_workspace_bytes(N, R, C, G, dtype);
+  const size_t need = streaming_only ? align_up(fwd_ws_bytes(N, R, C, G, dtype, true), 256) : gnnhwc_fwd_workspace_bytes(N, R, C, G, dtype);
   if (!workspace || !aligned16(workspace) || workspace_bytes < need)
     return fail(GNNHWC_ERR_WORKSPACE, "forward workspace must be 16-byte aligned and at least %zu bytes (got %p, %zu bytes)",
                 need, workspace, workspace_bytes);
   const int vec = 16 / elem_size(dtype);
   const bool vector_ok = C % vec == 0 && aligned16(x) && aligned16(y) && aligned16(add.residual) && aligned16(add.sum_out);
   FwdArgs a;
+  a.streaming_only = streaming_only;
   a.add = add;
   a.x = x; a.w = weight; a.b = bias; a.y = y; a.mean = mean; a.rstd = rstd;
   a.eps = eps; a.act = act; a.pdtype = param_dtype; a.sdtype = stats_dtype;
@@ -482,6 +523,37 @@ int gnnhwc_fwd(const void *x, const void *weight, const void *bias, void *y, voi
   const AddArgs none = {nullptr, nullptr, GN_F32, nullptr};
   return forward(x, none, weight, bias, y, mean, rstd, N, R, C, G, eps, act, dtype, param_dtype, stats_dtype, workspace,
                  workspace_bytes, stream);
+}
+
+size_t gnnhwc_fwd_static_scratch_bytes(int64_t N, int64_t R, int64_t C, int64_t G, int dtype) {
+  if (check_shape(N, R, C, G, dtype) != GNNHWC_OK) return 0;
+  if (N == 0 || R == 0) return 256;
+  return align_up(fwd_ws_bytes(N, R, C, G, dtype, true), 256);
+}
+
+int gnnhwc_fwd_static(const void *x, const void *weight, const void *bias, void *y, void *mean, void *rstd, int64_t N,
+                      int64_t R, int64_t C, int64_t G, double eps, int act, int dtype, int param_dtype, int stats_dtype,
+                      void *stream) {
+  int rc = check_shape(N, R, C, G, dtype);
+  if (rc != GNNHWC_OK) return rc;
+  void *ptr = nullptr;
+  if (N > 0 && R > 0) {  // (an empty problem launches nothing and needs no scratch; its other arguments are still checked)
+    const size_t need = gnnhwc_fwd_static_scratch_bytes(N, R, C, G, dtype);
+    if (need > (size_t)GNNHWC_STATIC_SCRATCH_BYTES)
+      return fail(GNNHWC_ERR_WORKSPACE,
+                  "gnnhwc_fwd_static: this problem needs %zu bytes of scratch memory, the library's own holds %zu; use "
+                  "gnnhwc_fwd with a caller-provided workspace", need, (size_t)GNNHWC_STATIC_SCRATCH_BYTES);
+    ptr = static_scratch();
+    if (!ptr) return GNNHWC_ERR_LAUNCH;
+  }
+  // no per-launch events here (creating one allocates): timing is off for the duration of this call
+  const bool profiling = g_profile;
+  g_profile = false;
+  const AddArgs none = {nullptr, nullptr, GN_F32, nullptr};
+  rc = forward(x, none, weight, bias, y, mean, rstd, N, R, C, G, eps, act, dtype, param_dtype, stats_dtype, ptr,
+               (size_t)GNNHWC_STATIC_SCRATCH_BYTES, stream, true);
+  g_profile = profiling;
+  return rc;
 }
 
 int gnnhwc_fwd_add(const void *x, const void *residual, const void *channel_bias, void *sum_out, const void *weight,

@@ -40,6 +40,7 @@ struct FwdArgs {
   void *ws;
   hipStream_t stream;
   Plan plan;
+  bool streaming_only = false;  // multi-launch kernels whatever the size (the entry point that must not allocate)
 };
 struct BwdArgs {
   const void *dy, *x, *w, *b, *mean, *rstd;

@@ -295,7 +295,7 @@ bool try_resident_bwd(const BwdArgs &a) {
 
 #if GN_PART_FWD
 template <int VEC> hipError_t fwd_impl(const FwdArgs &a) {
-  if (VEC != 1 && try_resident_fwd(a)) return hipGetLastError();
+  if (VEC != 1 && !a.streaming_only && try_resident_fwd(a)) return hipGetLastError();
   if (a.has_add()) {
     // multi-launch form: materialise the sum (in sum_out, or in y when the caller does not want it), then
     // normalise it from there (in place when it sits in y)

@@ -12,6 +12,7 @@ LIB_PATH = os.path.join(_CSRC, "libgnnhwc_hip.so")
 
 # dtype / activation codes of include/gnnhwc.h
 F32, F64, F16, BF16 = 0, 1, 2, 3
+STATIC_SCRATCH_BYTES = 4 << 20  # GNNHWC_STATIC_SCRATCH_BYTES
 NUM_KERNEL_KINDS = 15
 
 SYMBOLS = (
@@ -21,6 +22,8 @@ SYMBOLS = (
     "gnnhwc_bwd_workspace_bytes",
     "gnnhwc_fwd",
     "gnnhwc_fwd_add",
+    "gnnhwc_fwd_static",
+    "gnnhwc_fwd_static_scratch_bytes",
     "gnnhwc_bwd",
     "gnnhwc_nchw_workspace_bytes",
     "gnnhwc_fwd_nchw",
@@ -56,6 +59,10 @@ def _load():
     lib.gnnhwc_fwd.restype = ci
     lib.gnnhwc_fwd_add.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, dbl, ci, ci, ci, ci, ci, vp, sz, vp]
     lib.gnnhwc_fwd_add.restype = ci
+    lib.gnnhwc_fwd_static.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, dbl, ci, ci, ci, ci, vp]
+    lib.gnnhwc_fwd_static.restype = ci
+    lib.gnnhwc_fwd_static_scratch_bytes.argtypes = [i64, i64, i64, i64, ci]
+    lib.gnnhwc_fwd_static_scratch_bytes.restype = sz
     lib.gnnhwc_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, ci, ci, ci, ci, vp, sz, vp]
     lib.gnnhwc_bwd.restype = ci
     lib.gnnhwc_nchw_workspace_bytes.argtypes = [i64, i64, i64, i64, ci, ci]

@@ -126,6 +126,32 @@ int gnnhwc_fwd_add(const void *x, const void *residual, const void *channel_bias
                    void *workspace, size_t workspace_bytes, void *stream /* hipStream_t */);
 
 /*
+ * Forward that allocates nothing (no counterpart in the reference, whose host driver takes its scratch from the
+ * caching allocator on every call, gn_kernel.cu:461,530).  For callers that cannot allocate device memory or have
+ * nobody to allocate for them: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * Same results contract and arguments as gnnhwc_fwd without the workspace: the per-tile partial statistics live in
+ * GNNHWC_STATIC_SCRATCH_BYTES of device memory that is part of the library's image (every device the library runs on
+ * holds its own copy until the process ends; the first call on a device looks its address up, nothing is allocated
+ * then or later, and no event, host-pinned word or other library state is created).  It always runs the multi-launch
+ * kernels (statistics, then normalise + activation: x is read twice), whose scratch needs no clearing: every word a
+ * launch reads has been written by the launch before it in the same call.
+ *   - A problem whose partial statistics need more than the scratch holds is rejected with GNNHWC_ERR_WORKSPACE and
+ *     nothing is launched; gnnhwc_fwd_static_scratch_bytes tells how much a problem needs (0 for an invalid shape).
+ *   - All calls on one device share that device's scratch: calls that overlap in time on one device (two streams,
+ *     two host threads, two concurrently replayed graphs) race and give undefined statistics.  Calls that follow
+ *     each other on one stream are safe.
+ *   - Per-kernel timing (gnnhwc_profile_enable) is ignored by this entry point.
+ */
+#define GNNHWC_STATIC_SCRATCH_BYTES (4u << 20)
+size_t gnnhwc_fwd_static_scratch_bytes(int64_t N, int64_t R, int64_t C, int64_t G, int dtype);
+int gnnhwc_fwd_static(const void *x, const void *weight, const void *bias,
+                      void *y, void *mean, void *rstd,
+                      int64_t N, int64_t R, int64_t C, int64_t G,
+                      double eps, int act,
+                      int dtype, int param_dtype, int stats_dtype,
+                      void *stream /* hipStream_t */);
+
+/*
  * Backward: given dy and the forward's inputs and statistics, recomputes the activation gradient and
  * returns dx (N,R,C), dweight (C) and dbias (C).
  * Replaces run_gn_bwd_kernels<T> (gn_kernel.h:26-41; gn_kernel.cu:932-1055).
