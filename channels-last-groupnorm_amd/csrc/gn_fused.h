@@ -118,12 +118,15 @@ __device__ __forceinline__ int record_slot(const PartialGeo &q, int G, int n, in
   return __mul24(__mul24(col, G) + g, q.tiles) + t;
 }
 
+// What a result is replaced by when a wait expired: not a number, so that the call's output cannot pass for one.
+__device__ __forceinline__ float poison() { return __builtin_nanf(""); }
 // Collect the records of group g (all tiles of the chunks that hold a piece of it) with L lanes: each lane polls its
 // own records until they carry this call's epoch, kRecFast at a time (they stay in registers: the round trip that
-// finds them ready also brings their values), and hands (value0, value1, count) of each to body.  Returns false if
-// a wait expired: the lane's records are then not this call's, and the caller must not produce a plausible result.
+// finds them ready also brings their values), and hands (value0, value1, count) of each to body.  If a wait expires,
+// the lane's records are not this call's: body is handed NaN values first, so that whatever the caller accumulates
+// cannot pass for a result.
 template <typename BODY>
-__device__ __forceinline__ bool for_group_records(const SyncArea &s, __amdgpu_buffer_rsrc_t rb, const PartialGeo &q,
+__device__ __forceinline__ void for_group_records(const SyncArea &s, __amdgpu_buffer_rsrc_t rb, const PartialGeo &q,
                                                   const Plan &p, int64_t n, int g, bool valid, int L, int sl, BODY &&body) {
   int k_lo = 0, nk = 1;
   if (valid) group_chunks(q, p.D, g, k_lo, nk);
@@ -131,7 +134,6 @@ __device__ __forceinline__ bool for_group_records(const SyncArea &s, __amdgpu_bu
   const int base = record_slot(q, p.G, (int)n, 0, k_lo, g);
   const int kstride = __mul24(p.G, q.tiles);
   int spins = 0;
-  bool good = true;
   for (int e0 = sl; e0 < P; e0 += kRecFast * L) {
     u32x4 rec[kRecFast];
     bool have[kRecFast];
@@ -155,7 +157,7 @@ __device__ __forceinline__ bool for_group_records(const SyncArea &s, __amdgpu_bu
       if (ok) break;
       if (++spins > s.max_spins) {
         *s.status = s.epoch;
-        good = false;
+        body(poison(), poison(), 1.0f);
         break;
       }
       __builtin_amdgcn_s_sleep(2);
@@ -169,10 +171,7 @@ __device__ __forceinline__ bool for_group_records(const SyncArea &s, __amdgpu_bu
       }
     }
   }
-  return good;
 }
-// What a result is replaced by when a wait expired: not a number, so that the call's output cannot pass for one.
-__device__ __forceinline__ float poison() { return __builtin_nanf(""); }
 
 // ---------------------------------------------------------------------------------------------
 // Resident forward.  NV = register capacity in rows per lane.  Statistics follow the same definitions
@@ -276,25 +275,45 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
 #pragma unroll
   for (int j = 0; j < VEC; ++j) { mean[j] = (A)0; m2[j] = (A)0; }
   if (rows > 0) {
+    // One pass, taken row by row as the rows arrive: sums of the deviations from the lane's own first row (a value
+    // of the data, so nothing cancels: the pivot form of the moments) and of their squares.  Nothing but a few
+    // operations per channel is left to do once the last row is there.
+    A k[VEC], s1[VEC], s2[VEC];
+    LV::unpack(buf[0], k);
 #pragma unroll
-    for (int u = 0; u < NV; ++u) {
-      const A keep = u < rows ? (A)1 : (A)0;
-      A v[VEC];
-      LV::unpack(buf[u], v);
+    for (int j = 0; j < VEC; ++j) { s1[j] = (A)0; s2[j] = (A)0; }
+    if (rows == NV) {  // a full tile (all but the last tile of a sample): no masking of rows past the lane's last one
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) mean[j] += keep * v[j];
+      for (int u = 1; u < NV; ++u) {
+        A v[VEC];
+        LV::unpack(buf[u], v);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const A d = v[j] - k[j];
+          s1[j] += d;
+          s2[j] += d * d;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int u = 1; u < NV; ++u) {
+        const bool keep = u < rows;
+        A v[VEC];
+        LV::unpack(buf[u], v);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const A d = keep ? v[j] - k[j] : (A)0;
+          s1[j] += d;
+          s2[j] += d * d;
+        }
+      }
     }
     const A inv = fast_rcp((A)rows);
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) mean[j] *= inv;
-#pragma unroll
-    for (int u = 0; u < NV; ++u) {
-      const A keep = u < rows ? (A)1 : (A)0;
-      A v[VEC];
-      pin(buf[u]);
-      LV::unpack(buf[u], v);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) { const A d = v[j] - mean[j]; m2[j] += keep * d * d; }
+    for (int j = 0; j < VEC; ++j) {
+      const A dm = s1[j] * inv;
+      mean[j] = k[j] + dm;
+      m2[j] = s2[j] - s1[j] * dm;
     }
   }
   const __amdgpu_buffer_rsrc_t rb = record_buffer(sync);
@@ -320,14 +339,13 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
       const int g = l.g_lo + gi;
       // each lane folds its records about the mean of its first one ...
       A nl = (A)0, kl = (A)0, s1 = (A)0, s2 = (A)0;
-      const bool good = for_group_records(sync, rb, q, p, n, g, valid, L, sl, [&](float mu, float mm, float cnt) {
+      for_group_records(sync, rb, q, p, n, g, valid, L, sl, [&](float mu, float mm, float cnt) {
         if (nl == (A)0) kl = mu;
         const A d = mu - kl;
         nl += cnt;
         s1 += cnt * d;
         s2 += mm + cnt * d * d;
       });
-      if (!good) s1 = poison();  // reaches mean and rstd of the group, and through them every y of this tile
       const A inv = nl > (A)0 ? fast_rcp(nl) : (A)0;
       const A mean_l = kl + s1 * inv;
       const A m2_l = s2 - s1 * s1 * inv;
@@ -377,7 +395,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
 //   channel records : {S1, S2, epoch} per (n, tile, channel) of the whole tensor (they feed dgamma / dbeta)
 // ---------------------------------------------------------------------------------------------
 template <typename T, typename PT, int VEC, int ACT, int NV>
-__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 ? 4 : NV <= 8 ? 3 : NV <= 16 ? 2 : 1))) void fused_bwd_kernel(
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 ? 4 : NV <= 8 ? 3 : NV <= 22 ? 2 : 1))) void fused_bwd_kernel(
     const T *__restrict__ x, const T *__restrict__ dy, T *__restrict__ dx, const void *mean, const void *rstd, int sdtype,
     const void *w, const void *b, SyncArea sync_arg, void *dw, void *db, const void *mean_all, const void *rstd_all,
     int64_t n0, int64_t n_all, Plan p) {
@@ -522,11 +540,10 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
       const bool valid = gi < l.ng;
       const int g = l.g_lo + gi;
       A ta = (A)0, tb = (A)0;
-      const bool good = for_group_records(sync, rb, q, p, n, g, valid, L, sl, [&](float ra, float rbv, float) {
+      for_group_records(sync, rb, q, p, n, g, valid, L, sl, [&](float ra, float rbv, float) {
         ta += ra;
         tb += rbv;
       });
-      if (!good) ta = poison();  // reaches both coefficients of the group, and through them every dx of this tile
       segment_sum2(ta, tb, L);
       if (valid && sl == 0) {
         const A mu = sm_mu[gi];
@@ -600,7 +617,6 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
   trace_point(sync, 4);
   if (tail) {
     int spins = 0;
-    bool tail_good = true;
     for (int cb = l.tile * cpp; cb < l.wch; cb += p.tiles * cpp) {
       const bool first = cb == l.tile * cpp;
       const int cc = cb + tslot;
@@ -615,7 +631,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
         while (valid && nn >= n0 && (!record_ready(rec, sync.epoch) || sync.max_spins == kForcedTimeout)) {
           if (++spins > sync.max_spins) {
             *sync.status = sync.epoch;
-            tail_good = false;
+            t1 = poison();  // dgamma / dbeta of this channel say so
+            t2 = poison();
             break;
           }
           __builtin_amdgcn_s_sleep(2);
@@ -641,7 +658,6 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
             load_scalar<A>(rstd_all, nn * p.G + g, sdtype));
       }
       if (!valid) { t1 = (A)0; t2 = (A)0; }
-      if (!tail_good) { t1 = poison(); t2 = poison(); }  // a wait expired: dgamma / dbeta of these channels say so
       segment_sum2(t1, t2, TL);
       if (valid && tsl == 0) {
         if (dw) store_param<PT, A>(dw, c, t1);

@@ -269,7 +269,8 @@ template <typename PT, int ACT> bool try_resident_bwd_act(const BwdArgs &a) {
   const int most = a.plan.N < worthwhile_batches(a.plan, true) ? (int)a.plan.N : worthwhile_batches(a.plan, true);
   for (int b = 1; b <= most; ++b)
     if (try_resident_bwd_nv<PT, ACT, 4>(a, b) || try_resident_bwd_nv<PT, ACT, 8>(a, b) ||
-        try_resident_bwd_nv<PT, ACT, 16>(a, b) || try_resident_bwd_nv<PT, ACT, 32>(a, b))
+        try_resident_bwd_nv<PT, ACT, 16>(a, b) || try_resident_bwd_nv<PT, ACT, 22>(a, b) ||
+        try_resident_bwd_nv<PT, ACT, 32>(a, b))
       return true;
   return false;
 }
