@@ -9,10 +9,11 @@ inputs, outputs and workspaces already resident in HBM.  The timed region is K s
 torch.cuda.synchronize() calls.  Prints ONE JSON line:
 
   value        algorithmic GB/s of the timed region: (2 S fwd + 3 S bwd per shape) / time
-  roofline     the dominant launch (the kernel kind and shape with the longest mean duration): its algorithmic
-               bytes / its mean duration, measured here with HIP events recorded on the launch stream around
-               every launch, against 8 TB/s; `traffic` is read from profiles/hbm_traffic_sd_unet.txt (rocprofv3
-               --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --counter-workload`), null when that file is absent
+  roofline     the dominant kernel (the kernel kind and shape the step spends the largest share of its kernel time
+               in: mean launch duration x launches per step): its algorithmic bytes / its mean duration, measured
+               here with HIP events bound to every launch on the launch stream, against 8 TB/s; every kernel's share
+               and fraction is listed under `kernels`; `traffic` is read from profiles/hbm_traffic_sd_unet.txt
+               (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --counter-workload`), null when absent
   copy_ceiling the library's plain copy kernel on tensors of each shape's size: what a kernel with no
                arithmetic and no cross-workgroup dependency reaches at that size on this GPU
   cpu_baseline torch.nn.functional.group_norm + SiLU + autograd on the host cores, same tensors (bounded sample)
@@ -333,7 +334,9 @@ def timeline(names, device, reps=5):
             time.sleep(0.002)
             rows = []
             for _ in range(reps):
-                p.step(0, stream, "both" if which == "bwd" else "fwd")  # a backward is measured behind its own forward, as in the sweep
+                p.step(0, stream, "both")  # the traced launch runs behind other kernels, as in the sweep: a backward behind its
+                if which == "fwd":         # own forward, a forward behind the backward of the call before
+                    p.step(0, stream, "fwd")
                 torch.cuda.synchronize()
                 _cabi.check(_cabi.lib.gnnhwc_debug_read_trace(words.ctypes.data, words.size), "gnnhwc_debug_read_trace")
                 t = words.astype(np.int64)
@@ -608,7 +611,11 @@ def main():
     def launch_bytes(name, kind):  # algorithmic bytes of ONE launch of this kind on this shape
         return KERNEL_STREAMS[kind] * S_of[name] / prof[name][kind][1]
 
-    dom_shape, dominant = max(((n, k) for n in prof for k in prof[n]), key=lambda nk: prof[nk[0]][nk[1]][0])
+    # time a kernel kind on a shape takes per step: mean launch duration x launches per call; the dominant kernel is
+    # the one the step spends most of its time in
+    step_us = {(n, k): prof[n][k][0] * prof[n][k][1] for n in prof for k in prof[n]}
+    total_us = sum(step_us.values())
+    dom_shape, dominant = max(step_us, key=step_us.get)
     dom_us = prof[dom_shape][dominant][0]
     dom_bytes = launch_bytes(dom_shape, dominant)
     achieved = dom_bytes / (dom_us * 1e-6) / 1e9
@@ -626,8 +633,11 @@ def main():
         "traffic_source": "profiles/hbm_traffic_sd_unet.txt (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, copy-calibrated)" if tr else None,
         "bytes_per_launch": dom_bytes,
         "mean_launch_us": round(dom_us, 3),
+        "share_of_step": round(step_us[(dom_shape, dominant)] / total_us, 4),
+        "selection": "largest share of the step's kernel time (mean launch duration x launches per step)",
         "kernels": {n: {k: {"us": round(us, 3), "launches_per_call": per_call, "alg_bytes": launch_bytes(n, k),
                             "frac": round(launch_bytes(n, k) / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+                            "share_of_step": round(step_us[(n, k)] / total_us, 4),
                             "traffic": (round(sum(traffic[(n, k)])) if (n, k) in traffic else None)}
                         for k, (us, per_call) in kinds.items()} for n, kinds in prof.items()},
     }
