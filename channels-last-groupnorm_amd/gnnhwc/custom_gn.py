@@ -6,6 +6,9 @@ reference; the kernels behind the operators are the HIP ones in libgnnhwc_hip.so
 C ABI (include/gnnhwc.h) with raw device pointers and the current HIP stream.  torch only provides
 device memory (outputs, workspace) and the stream.
 """
+import collections
+import threading
+
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
@@ -56,6 +59,25 @@ def _as_nrc(t):
     return t if t.is_contiguous() else t.contiguous()
 
 
+def _param_args(weight, bias, C, data_code):
+    """(param dtype code, weight pointer, bias pointer, tensors to keep alive) for the C ABI.  weight and bias are
+    either both tensors of C elements on the device and of one dtype, or both None: the C ABI takes NULL for
+    gamma = 1, beta = 0, so a normalisation without parameters never materialises ones and zeros
+    (the reference does, custom_gn.py:83-86)."""
+    if weight is None and bias is None:
+        return data_code, None, None, ()
+    if weight is None or bias is None:
+        raise RuntimeError("weight and bias must both be given or both be None")
+    _check_device(weight, "weight")
+    _check_device(bias, "bias")
+    if bias.dtype != weight.dtype:
+        raise RuntimeError("weight and bias must have the same dtype (%s vs %s)" % (weight.dtype, bias.dtype))
+    if weight.numel() != C or bias.numel() != C:
+        raise RuntimeError("weight and bias must have %d elements" % C)
+    w, b = weight.contiguous(), bias.contiguous()
+    return _dtype_code(weight, "weight"), w.data_ptr(), b.data_ptr(), (w, b)
+
+
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
@@ -86,37 +108,40 @@ class _on_device:
         return False
 
 
-_workspaces = {}
+_workspaces = collections.OrderedDict()
+_workspaces_lock = threading.Lock()
+_MAX_CACHED_WORKSPACES = 8
 
 
 def _workspace(nbytes, device, stream_ptr):
     """Scratch memory for one call.  Calls on one stream follow each other, so they can share one buffer per
     (device, stream), grown on demand; while the stream is recording a graph the buffer comes from the allocator
-    instead (it then belongs to the graph's own memory pool, like every other tensor of the capture)."""
+    instead (it then belongs to the graph's own memory pool, like every other tensor of the capture).
+    The cache is shared by the caller's thread and the autograd engine's, hence the lock; it keeps the buffers of the
+    most recently used streams only, so that streams that no longer exist do not pin memory for ever (a buffer that is
+    dropped while a kernel still uses it stays valid: the caching allocator only reuses it in stream order)."""
     if torch.cuda.is_current_stream_capturing():
         return torch.empty((nbytes,), dtype=torch.uint8, device=device)
     key = (device.index, stream_ptr)
-    ws = _workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.empty((max(nbytes, 1 << 20),), dtype=torch.uint8, device=device)
-        _workspaces[key] = ws
+    with _workspaces_lock:
+        ws = _workspaces.get(key)
+        if ws is None or ws.numel() < nbytes:
+            ws = torch.empty((max(nbytes, 1 << 20),), dtype=torch.uint8, device=device)
+            _workspaces[key] = ws
+        _workspaces.move_to_end(key)
+        while len(_workspaces) > _MAX_CACHED_WORKSPACES:
+            _workspaces.popitem(last=False)
     return ws
 
 
 def gn_nhwc_fwd(X, weight, bias, G, eps, act_fn_option):
     """gnop::fwd -- custom_gn.cpp:10-42.  X: (N, C, R) channels-last view.  Returns (Y, means, rstds)."""
     _check_device(X, "X")
-    _check_device(weight, "weight")
-    _check_device(bias, "bias")
     if X.dim() != 3:
         raise RuntimeError("gnop::fwd expects X of shape (N, C, R), got %s" % (tuple(X.shape),))
     N, C, R = X.shape
     dt = _dtype_code(X, "X")
-    pdt = _dtype_code(weight, "weight")
-    if bias.dtype != weight.dtype:
-        raise RuntimeError("weight and bias must have the same dtype (%s vs %s)" % (weight.dtype, bias.dtype))
-    if weight.numel() != C or bias.numel() != C:
-        raise RuntimeError("weight and bias must have %d elements" % C)
+    pdt, w_ptr, b_ptr, _keep = _param_args(weight, bias, C, dt)
     X_nrc = _as_nrc(X)
     Y = torch.empty_like(X_nrc)
     sdtype = _stats_dtype(X.dtype)
@@ -130,7 +155,7 @@ def gn_nhwc_fwd(X, weight, bias, G, eps, act_fn_option):
         stream = _current_stream_ptr(X.device)
         ws = _workspace(nbytes, X.device, stream)
         rc = lib.gnnhwc_fwd(
-            X_nrc.data_ptr(), weight.contiguous().data_ptr(), bias.contiguous().data_ptr(),
+            X_nrc.data_ptr(), w_ptr, b_ptr,
             Y.data_ptr(), means.data_ptr(), rstds.data_ptr(),
             N, R, C, G, float(eps), int(act_fn_option), dt, pdt, _DTYPE_CODE[sdtype],
             ws.data_ptr(), ws.numel(), stream)
@@ -140,26 +165,27 @@ def gn_nhwc_fwd(X, weight, bias, G, eps, act_fn_option):
 
 def gn_nhwc_bwd(dy, X, weight, bias, means, rstds, G, act_fn_option):
     """gnop::bwd -- custom_gn.cpp:44-89.  Returns (dX (N, C, R) channels-last view, dweight, dbias)."""
-    for t, name in ((dy, "dy"), (X, "X"), (weight, "weight"), (bias, "bias"), (means, "means"), (rstds, "rstds")):
+    for t, name in ((dy, "dy"), (X, "X"), (means, "means"), (rstds, "rstds")):
         _check_device(t, name)
     if X.dim() != 3 or dy.shape != X.shape:
         raise RuntimeError("gnop::bwd expects dy and X of the same shape (N, C, R), got %s and %s"
                            % (tuple(dy.shape), tuple(X.shape)))
     N, C, R = X.shape
     dt = _dtype_code(X, "X")
-    pdt = _dtype_code(weight, "weight")
+    pdt, w_ptr, b_ptr, _keep = _param_args(weight, bias, C, dt)
     sdt = _dtype_code(means, "means")
     if dy.dtype != X.dtype:
         raise RuntimeError("dy and X must have the same dtype (%s vs %s)" % (dy.dtype, X.dtype))
-    if rstds.dtype != means.dtype or bias.dtype != weight.dtype:
-        raise RuntimeError("means/rstds and weight/bias must pairwise share a dtype")
+    if rstds.dtype != means.dtype:
+        raise RuntimeError("means and rstds must share a dtype")
     if means.numel() != N * G or rstds.numel() != N * G:
         raise RuntimeError("means and rstds must have N*G = %d elements" % (N * G))
     X_nrc = _as_nrc(X)
     dy_nrc = _as_nrc(dy)
     dX = torch.empty_like(X_nrc)
-    dweight = torch.empty((C,), dtype=weight.dtype, device=X.device)
-    dbias = torch.empty((C,), dtype=weight.dtype, device=X.device)
+    # a normalisation without parameters has no parameter gradients: nothing is allocated or computed for them
+    dweight = torch.empty((C,), dtype=weight.dtype, device=X.device) if weight is not None else None
+    dbias = torch.empty((C,), dtype=bias.dtype, device=X.device) if bias is not None else None
     lib = _cabi.lib
     with _on_device(X.device):
         nbytes = lib.gnnhwc_bwd_workspace_bytes(N, R, C, G, dt)
@@ -168,9 +194,9 @@ def gn_nhwc_bwd(dy, X, weight, bias, means, rstds, G, act_fn_option):
         stream = _current_stream_ptr(X.device)
         ws = _workspace(nbytes, X.device, stream)
         rc = lib.gnnhwc_bwd(
-            dy_nrc.data_ptr(), X_nrc.data_ptr(), weight.contiguous().data_ptr(), bias.contiguous().data_ptr(),
+            dy_nrc.data_ptr(), X_nrc.data_ptr(), w_ptr, b_ptr,
             means.contiguous().data_ptr(), rstds.contiguous().data_ptr(),
-            dX.data_ptr(), dweight.data_ptr(), dbias.data_ptr(),
+            dX.data_ptr(), dweight.data_ptr() if dweight is not None else None, dbias.data_ptr() if dbias is not None else None,
             N, R, C, G, int(act_fn_option), dt, pdt, sdt,
             ws.data_ptr(), ws.numel(), stream)
     _cabi.check(rc, "gnop::bwd")
@@ -181,17 +207,11 @@ def gn_nchw_fwd(X, weight, bias, G, eps, act_fn_option):
     """gnop::fwd_nchw (no counterpart in the reference, which hands channels-first input to torch,
     custom_gn.py:75-79): X is (N, C, R) contiguous.  Returns (Y contiguous like X, means, rstds)."""
     _check_device(X, "X")
-    _check_device(weight, "weight")
-    _check_device(bias, "bias")
     if X.dim() != 3:
         raise RuntimeError("gnop::fwd_nchw expects X of shape (N, C, R), got %s" % (tuple(X.shape),))
     N, C, R = X.shape
     dt = _dtype_code(X, "X")
-    pdt = _dtype_code(weight, "weight")
-    if bias.dtype != weight.dtype:
-        raise RuntimeError("weight and bias must have the same dtype (%s vs %s)" % (weight.dtype, bias.dtype))
-    if weight.numel() != C or bias.numel() != C:
-        raise RuntimeError("weight and bias must have %d elements" % C)
+    pdt, w_ptr, b_ptr, _keep = _param_args(weight, bias, C, dt)
     X = X.contiguous()
     Y = torch.empty_like(X)
     sdtype = _stats_dtype(X.dtype)
@@ -205,7 +225,7 @@ def gn_nchw_fwd(X, weight, bias, G, eps, act_fn_option):
         stream = _current_stream_ptr(X.device)
         ws = _workspace(nbytes, X.device, stream)
         rc = lib.gnnhwc_fwd_nchw(
-            X.data_ptr(), weight.contiguous().data_ptr(), bias.contiguous().data_ptr(),
+            X.data_ptr(), w_ptr, b_ptr,
             Y.data_ptr(), means.data_ptr(), rstds.data_ptr(),
             N, C, R, G, float(eps), int(act_fn_option), dt, pdt, _DTYPE_CODE[sdtype],
             ws.data_ptr(), ws.numel(), stream)
@@ -215,26 +235,26 @@ def gn_nchw_fwd(X, weight, bias, G, eps, act_fn_option):
 
 def gn_nchw_bwd(dy, X, weight, bias, means, rstds, G, act_fn_option):
     """gnop::bwd_nchw: dy, X (N, C, R) contiguous.  Returns (dX, dweight, dbias)."""
-    for t, name in ((dy, "dy"), (X, "X"), (weight, "weight"), (bias, "bias"), (means, "means"), (rstds, "rstds")):
+    for t, name in ((dy, "dy"), (X, "X"), (means, "means"), (rstds, "rstds")):
         _check_device(t, name)
     if X.dim() != 3 or dy.shape != X.shape:
         raise RuntimeError("gnop::bwd_nchw expects dy and X of the same shape (N, C, R), got %s and %s"
                            % (tuple(dy.shape), tuple(X.shape)))
     N, C, R = X.shape
     dt = _dtype_code(X, "X")
-    pdt = _dtype_code(weight, "weight")
+    pdt, w_ptr, b_ptr, _keep = _param_args(weight, bias, C, dt)
     sdt = _dtype_code(means, "means")
     if dy.dtype != X.dtype:
         raise RuntimeError("dy and X must have the same dtype (%s vs %s)" % (dy.dtype, X.dtype))
-    if rstds.dtype != means.dtype or bias.dtype != weight.dtype:
-        raise RuntimeError("means/rstds and weight/bias must pairwise share a dtype")
+    if rstds.dtype != means.dtype:
+        raise RuntimeError("means and rstds must share a dtype")
     if means.numel() != N * G or rstds.numel() != N * G:
         raise RuntimeError("means and rstds must have N*G = %d elements" % (N * G))
     X = X.contiguous()
     dy = dy.contiguous()
     dX = torch.empty_like(X)
-    dweight = torch.empty((C,), dtype=weight.dtype, device=X.device)
-    dbias = torch.empty((C,), dtype=weight.dtype, device=X.device)
+    dweight = torch.empty((C,), dtype=weight.dtype, device=X.device) if weight is not None else None
+    dbias = torch.empty((C,), dtype=bias.dtype, device=X.device) if bias is not None else None
     lib = _cabi.lib
     with _on_device(X.device):
         nbytes = lib.gnnhwc_nchw_workspace_bytes(N, C, R, G, dt, 1)
@@ -243,9 +263,9 @@ def gn_nchw_bwd(dy, X, weight, bias, means, rstds, G, act_fn_option):
         stream = _current_stream_ptr(X.device)
         ws = _workspace(nbytes, X.device, stream)
         rc = lib.gnnhwc_bwd_nchw(
-            dy.data_ptr(), X.data_ptr(), weight.contiguous().data_ptr(), bias.contiguous().data_ptr(),
+            dy.data_ptr(), X.data_ptr(), w_ptr, b_ptr,
             means.contiguous().data_ptr(), rstds.contiguous().data_ptr(),
-            dX.data_ptr(), dweight.data_ptr(), dbias.data_ptr(),
+            dX.data_ptr(), dweight.data_ptr() if dweight is not None else None, dbias.data_ptr() if dbias is not None else None,
             N, C, R, G, int(act_fn_option), dt, pdt, sdt,
             ws.data_ptr(), ws.numel(), stream)
     _cabi.check(rc, "gnop::bwd_nchw")
@@ -348,7 +368,7 @@ def _fwd_add_meta(X, residual, channel_bias, weight, bias, G, eps, act_fn_option
 
 
 # The reference's operators cannot be traced (its forward is wrapped in torch._dynamo.disable, custom_gn.py:63);
-# with these the operators at least carry correct output metadata under fake-tensor tracing.
+# with these the operators carry correct output metadata under fake-tensor tracing.
 _op_lib.impl("fwd", _fwd_meta, "Meta")
 _op_lib.impl("bwd", _bwd_meta, "Meta")
 _op_lib.impl("fwd_add", _fwd_add_meta, "Meta")
@@ -390,6 +410,15 @@ def _fwd_backward(ctx, dY, _dmeans, _drstds):
 # Autograd formula of gnop::fwd itself (the reference only differentiates through GN_NHWC_Func, custom_gn.py:29-47):
 # with it and the meta kernels above, code that calls the operator directly can be traced and compiled whole.
 torch.library.register_autograd("gnop::fwd", _fwd_backward, setup_context=_fwd_setup_context, lib=_op_lib)
+
+
+def _fwd_nchw_backward(ctx, dY, _dmeans, _drstds):
+    X, weight, bias, means, rstds = ctx.saved_tensors
+    dX, dweight, dbias = torch.ops.gnop.bwd_nchw(dY.contiguous(), X, weight, bias, means, rstds, ctx.G, ctx.act_fn_option)
+    return dX, dweight, dbias, None, None, None
+
+
+torch.library.register_autograd("gnop::fwd_nchw", _fwd_nchw_backward, setup_context=_fwd_setup_context, lib=_op_lib)
 
 
 def _fwd_add_setup_context(ctx, inputs, output):
@@ -540,8 +569,12 @@ class GN_NHWC(nn.GroupNorm):
         self.activation = activation
         self.act_code = ACTIVATION_CODES[activation]  # unknown name -> KeyError, as in the reference
 
-    @torch._dynamo.disable
     def forward(self, x):
+        # The reference wraps this method in torch._dynamo.disable (custom_gn.py:63): its operators cannot be traced,
+        # so a compiled model breaks its graph here.  These operators can (meta kernels + registered autograd), so
+        # under torch.compile the same computation is expressed through them and stays inside the caller's graph.
+        if torch.compiler.is_compiling():
+            return self._forward_traced(x)
         if x.stride(1) == 1:
             # channels fastest.  Make the remaining dims contiguous in their logical order as well: a shape
             # (2, 3, 5, 9) input must have strides (135, 1, 27, 3), not e.g. (135, 1, 3, 15) (custom_gn.py:68-73).
@@ -563,12 +596,29 @@ class GN_NHWC(nn.GroupNorm):
                 def run(t, w, b, g, eps, _code):
                     return act(F.group_norm(t, g, w, b, eps))
 
+        # affine=False: the reference materialises ones and zeros on every call (custom_gn.py:83-86); here the absent
+        # parameters travel as None down to the kernels, which take NULL for gamma = 1, beta = 0
+        return run(x, self.weight, self.bias, self.num_groups, self.eps, self.act_code)
+
+    def _forward_traced(self, x):
+        """forward() as torch.compile sees it: the same kernels through torch.ops.gnop.*, whose schemas take
+        tensors only, so a normalisation without parameters passes ones and zeros here."""
+        C = self.num_channels
         if self.affine:
             w, b = self.weight, self.bias
-        else:  # custom_gn.py:83-86
-            w = torch.ones((self.num_channels,), device=x.device, dtype=x.dtype)
-            b = torch.zeros((self.num_channels,), device=x.device, dtype=x.dtype)
-        return run(x, w, b, self.num_groups, self.eps, self.act_code)
+        else:
+            w, b = x.new_ones((C,)), x.new_zeros((C,))
+        if not x.is_cuda:
+            return _TORCH_ACTIVATIONS[self.act_code](F.group_norm(x.contiguous(), self.num_groups, w, b, self.eps))
+        if x.stride(1) == 1:
+            return group_norm_nhwc(x, w, b, self.num_groups, self.eps, self.activation)
+        shape = x.shape
+        R = 1
+        for d in shape[2:]:
+            R *= d
+        Y, _means, _rstds = torch.ops.gnop.fwd_nchw(x.contiguous().view(shape[0], C, R), w, b, self.num_groups, self.eps,
+                                                    self.act_code)
+        return Y.view(shape)
 
     def extra_repr(self):
         return "{num_groups}, {num_channels}, eps={eps}, affine={affine}, activation={activation}".format(**self.__dict__)

@@ -68,9 +68,12 @@ def check_against_torch(x, G, act, w, b, dy, eps=1e-5, relu_band=1e-4):
         if dtype == torch.float64:
             assert e <= TOL[dtype], "%s: err %.3g" % (k, e)
         elif dtype == torch.float32:
-            # 1e-5, or -- for ill-conditioned cases such as two-element groups -- within twice torch's own fp32
-            # error against the same truth (the reference's second-stage rule, test/check_outputs.py:134)
-            assert e <= TOL[dtype] or e <= 2 * err(l, t), "%s: err %.3g, torch fp32 %.3g" % (k, e, err(l, t))
+            # 1e-5; only for ill-conditioned slabs of at most four elements per group (two equal values make the
+            # variance vanish) also within twice torch's own fp32 error against the same truth (the reference's
+            # second-stage rule, test/check_outputs.py:134)
+            per_group = x.numel() // (x.shape[0] * G)
+            ok = e <= TOL[dtype] or (per_group <= 4 and e <= 2 * err(l, t))
+            assert ok, "%s: err %.3g, torch fp32 %.3g, %d elements per group" % (k, e, err(l, t), per_group)
         else:
             e_lib = err(l, t)
             assert e <= e_lib * (1 + HALF_SLACK) + 1e-12, "%s: err %.3g vs torch's own %.3g" % (k, e, e_lib)
@@ -209,11 +212,20 @@ def test_nchw_nhwc_equal(family, device):
             out1, out2 = m(a), m(c)
             out1.backward(rand_dy.to(dtype))
             out2.backward(rand_dy_nhwc.to(dtype))
-            # the reference's bound (1e-6) holds for f16 / f32 / f64; two bf16 results that differ in the last bit
-            # of some elements (the two kernel families sum in different orders) are bounded by 1e-4 instead.
-            bound = 1e-4 if dtype == torch.bfloat16 else 1e-6
-            assert (out1 - out2).float().square().mean() < bound
-            assert (a.grad - c.grad).float().square().mean() < bound
+            if dtype != torch.bfloat16:
+                # the reference's bound
+                assert (out1 - out2).float().square().mean() < 1e-6
+                assert (a.grad - c.grad).float().square().mean() < 1e-6
+            else:
+                # two bf16 results may differ in the last bit of some elements (the two kernel families sum in
+                # different orders), which already exceeds 1e-6 in the mean square; each layout is held to the
+                # half-precision rule instead: no further from the float64 truth than torch's own bf16 result
+                w, b = m.weight.detach(), m.bias.detach()
+                truth = orc.torch_reference(x.double(), w.double(), b.double(), G, m.eps, act, rand_dy.double())
+                lib = orc.torch_reference(x.to(dtype), w, b, G, m.eps, act, rand_dy.to(dtype))
+                for got_y, got_dx in ((out1, a.grad), (out2, c.grad)):
+                    assert err(got_y.double(), truth["y"]) <= err(lib["y"].double(), truth["y"]) * (1 + HALF_SLACK)
+                    assert err(got_dx.double(), truth["dx"]) <= err(lib["dx"].double(), truth["dx"]) * (1 + HALF_SLACK)
 
 
 @pytest.mark.parametrize("name", ["c5a_fp32_silu", "c5b_fp32_gelu", "c5c_fp32_relu", "c2", "c3b"])
@@ -596,6 +608,125 @@ def test_functional_form_traces_into_one_graph(dtype, device):
     assert y2.stride() == y.stride()
     gx2, gw2, gb2 = torch.autograd.grad(y2, (x2, w2, b2), dy)
     assert torch.equal(y2, y) and torch.equal(gx2, gx) and torch.equal(gw2, gw) and torch.equal(gb2, gb)
+
+
+@pytest.mark.gpu
+def test_non_affine_module_materialises_no_parameters(device, monkeypatch):
+    """affine=False: the reference fills a ones and a zeros tensor on every call (custom_gn.py:83-86); here the absent
+    parameters reach the kernels as NULL.  Same bits as the affine module with weight 1 and bias 0, no parameter
+    gradients, and no call of torch.ones / torch.zeros during forward or backward."""
+    gen = torch.Generator().manual_seed(9)
+    for shape, layout in (((2, 48, 9, 9), "last"), ((2, 48, 9, 9), "first")):
+        x = channels_last_like(shape, torch.bfloat16, device, gen, 1.5, 0.2)
+        dy = channels_last_like(shape, torch.bfloat16, device, gen)
+        if layout == "first":
+            x, dy = x.contiguous(), dy.contiguous()
+        m_ref = GN_NHWC(6, 48, activation="gelu").to(device).to(torch.bfloat16)
+        m = GN_NHWC(6, 48, activation="gelu", affine=False).to(device).to(torch.bfloat16)
+        xr = x.clone().requires_grad_(True)
+        want = m_ref(xr)
+        want.backward(dy)
+
+        def forbidden(*a, **k):
+            raise AssertionError("a ones / zeros tensor was materialised")
+
+        xa = x.clone().requires_grad_(True)
+        with monkeypatch.context() as mp:
+            mp.setattr(torch, "ones", forbidden)
+            mp.setattr(torch, "zeros", forbidden)
+            got = m(xa)
+            got.backward(dy)
+        assert torch.equal(got, want) and torch.equal(xa.grad, xr.grad)
+        assert m.weight is None and m.bias is None
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("xdtype", [torch.bfloat16, torch.float16])
+def test_module_with_float32_parameters_and_16_bit_input(family, xdtype, device):
+    """The autocast / AMP case the reference cannot run (it reads weight as the data type, custom_gn.cpp:35-36): a module
+    whose parameters stay float32 while x arrives in a 16-bit type, with and without torch.autocast around the call.
+    y and dx come back in x's type, dweight / dbias in float32.  Truth: the float64 oracle on the same values; y / dx
+    within half a spacing of the 16-bit type of it (one rounding of a float32-accurate value), dweight / dbias to the
+    float32 bar scaled by the 16-bit rounding of dy * act' that autograd's own chain would apply too."""
+    gen = torch.Generator().manual_seed(31)
+    shape, G = (2, 64, 20, 12), 8
+    x = channels_last_like(shape, xdtype, device, gen, 1.7, 0.4)
+    dy = channels_last_like(shape, xdtype, device, gen)
+    m = GN_NHWC(G, shape[1], activation="silu").to(device)  # float32 parameters
+    with torch.no_grad():
+        m.weight.copy_(torch.rand(shape[1], generator=gen) + 0.5)
+        m.bias.copy_(0.1 * torch.randn(shape[1], generator=gen))
+    truth = orc.fwd_bwd(orc.to_nrc(x), m.weight.detach().double().cpu().numpy(), m.bias.detach().double().cpu().numpy(),
+                        orc.to_nrc(dy), G, m.eps, orc.ACT_CODES["silu"])
+    half = 2.0 ** -8 if xdtype == torch.bfloat16 else 2.0 ** -11
+
+    def close_16(got, want):
+        t = torch.as_tensor(want)
+        d = (torch.as_tensor(orc.to_nrc(got)) - t).abs()
+        return bool((d <= half * 1.001 * t.abs() + 1e-5 * (t.abs() + float(t.square().mean().sqrt())) + 2.0 ** -24).all())
+
+    for use_autocast in (False, True):
+        m.zero_grad()
+        xr = x.clone().requires_grad_(True)
+        if use_autocast:
+            with torch.autocast(device_type="cuda", dtype=xdtype):
+                y = m(xr)
+        else:
+            y = m(xr)
+        y.backward(dy)
+        assert y.dtype == xdtype and xr.grad.dtype == xdtype
+        assert m.weight.grad.dtype == torch.float32 and m.bias.grad.dtype == torch.float32
+        assert close_16(y, truth["y"]), "y (autocast=%s)" % use_autocast
+        # dx carries one more 16-bit rounding: the single-launch backward keeps dy * act'(z) in x's type between its two
+        # phases (the rounding an unfused activation backward applies to the same quantity)
+        assert err(xr.grad, orc.from_nrc(truth["dx"], shape)) <= 3 * half, "dx (autocast=%s)" % use_autocast
+        assert err(m.weight.grad, truth["dw"]) <= 1e-5 and err(m.bias.grad, truth["db"]) <= 1e-5
+
+
+class _Block(nn.Module):
+    """A layer either side of the norm, so that a compiled graph has something of its own to fuse around the operator
+    (scalings by powers of two: exact in any type and any evaluation order)."""
+
+    def __init__(self, G, C, act, affine=True):
+        super().__init__()
+        self.norm = GN_NHWC(G, C, activation=act, affine=affine)
+
+    def forward(self, x):
+        return self.norm(x * 2.0) * 0.5
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("backend", ["aot_eager", "inductor"])
+def test_model_with_the_module_compiles_whole(backend, device):
+    """torch.compile of a model that contains GN_NHWC itself (the reference's forward is a guaranteed graph break,
+    custom_gn.py:63): fullgraph=True, so a break is an error; with the default backend (inductor) and with the tracing
+    one.  Outputs and all gradients equal the eager module's bit for bit, for channels-last and channels-first input,
+    with and without parameters."""
+    gen = torch.Generator().manual_seed(17)
+    shape, G = (2, 64, 16, 16), 8
+    for dtype, layout, affine in ((torch.float32, "last", True), (torch.bfloat16, "last", True),
+                                  (torch.bfloat16, "first", True), (torch.float32, "last", False)):
+        x0 = channels_last_like(shape, dtype, device, gen, 1.3, 0.2)
+        dy = channels_last_like(shape, dtype, device, gen)
+        if layout == "first":
+            x0, dy = x0.contiguous(), dy.contiguous()
+        model = _Block(G, shape[1], "silu", affine).to(device=device, dtype=dtype)
+        if affine:
+            with torch.no_grad():
+                model.norm.weight.copy_((torch.rand(shape[1], generator=gen) + 0.5).to(dtype))
+                model.norm.bias.copy_((0.1 * torch.randn(shape[1], generator=gen)).to(dtype))
+        params = list(model.parameters())
+        x = x0.clone().requires_grad_()
+        y = model(x)
+        want = torch.autograd.grad(y, [x] + params, dy)
+        torch._dynamo.reset()
+        compiled = torch.compile(model, backend=backend, fullgraph=True)
+        x2 = x0.clone().requires_grad_()
+        y2 = compiled(x2)
+        got = torch.autograd.grad(y2, [x2] + params, dy)
+        assert torch.equal(y2, y), (backend, dtype, layout, affine)
+        for g, w in zip(got, want):
+            assert torch.equal(g, w), (backend, dtype, layout, affine)
 
 
 @pytest.mark.gpu
