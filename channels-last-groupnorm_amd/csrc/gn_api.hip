@@ -702,6 +702,9 @@ static int nchw_call(NchwArgs &a, int dtype, void *workspace, size_t workspace_b
   const int64_t chunks = (a.R + nchw_chunk_len(vec) - 1) / nchw_chunk_len(vec);
   if ((double)a.N * (double)a.C * (double)chunks / 4.0 > 2.0e9)
     return fail(GNNHWC_ERR_INVALID_ARGUMENT, "%s: too many rows for one launch (N C = %lld)", what, (long long)(a.N * a.C));
+  if ((double)(a.C / a.G) * (double)chunks >= 2147483648.0)
+    return fail(GNNHWC_ERR_INVALID_ARGUMENT, "%s: a group of %lld rows of %lld elements is beyond the supported range", what,
+                (long long)(a.C / a.G), (long long)a.R);
   a.ws = workspace;
   hipError_t e;
   switch (dtype) {

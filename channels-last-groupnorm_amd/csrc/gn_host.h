@@ -65,10 +65,15 @@ struct NchwArgs {
 };
 // Elements of one chunk of a channel row: 64 lanes x vec elements x 4 lane vectors (kNchwUnroll in gn_nchw.h).
 inline int nchw_chunk_len(int vec) { return 64 * vec * 4; }
-// Accumulation-type elements of workspace: 3 planes forward, 2 backward, of [N * C][chunks].
-inline size_t nchw_workspace_elems(int64_t N, int64_t C, int64_t R, int vec, bool backward) {
+// Accumulation-type elements of the per-chunk partials: 3 planes forward, 2 backward, of [N * C][chunks] ...
+inline size_t nchw_partial_elems(int64_t N, int64_t C, int64_t R, int vec, bool backward) {
   const int64_t chunks = (R + nchw_chunk_len(vec) - 1) / nchw_chunk_len(vec);
-  return (size_t)(backward ? 2 : 3) * (size_t)(N * C * chunks);
+  return ((size_t)(backward ? 2 : 3) * (size_t)(N * C * chunks) + 63) / 64 * 64;
+}
+// ... and of the whole workspace: behind them, 2 planes [N * G] for the per-slab records of the compaction launch
+// (at most N * C elements each, whatever G is).
+inline size_t nchw_workspace_elems(int64_t N, int64_t C, int64_t R, int vec, bool backward) {
+  return nchw_partial_elems(N, C, R, vec, backward) + 2 * (size_t)(N * C);
 }
 
 // Workspace layout, in elements of the accumulation type (float, or double for f64 data).

@@ -102,9 +102,9 @@ __device__ __forceinline__ void nchw_merge_slab(const A *__restrict__ part, cons
                                                 A &mean, A &m2) {
   const int64_t plane = q.rows * q.chunks;
   const int64_t first = (n * q.C + (int64_t)g * q.D) * q.chunks;
-  const int P = q.D * q.chunks;
+  const int64_t P = (int64_t)q.D * q.chunks;
   A nl = (A)0, kl = (A)0, s1 = (A)0, s2 = (A)0;
-  for (int i = lane; i < P; i += 64) {
+  for (int64_t i = lane; i < P; i += 64) {
     const A cn = part[first + i], mu = part[plane + first + i], mm = part[2 * plane + first + i];
     if (nl == (A)0) kl = mu;
     const A d = mu - kl;
@@ -125,14 +125,65 @@ __device__ __forceinline__ void nchw_merge_slab(const A *__restrict__ part, cons
   m2 = t2 - t1 * dm;
 }
 
+// A slab has D * chunks partials and as many wavefronts, each of which needs the slab's merged result: merged by every
+// wavefront in its own prologue that is D * chunks reads per wavefront, fine for the usual few dozen (one launch
+// saved) and quadratic for one group of many long rows.  Beyond kNchwMergeInline partials per slab a compaction launch
+// of one wavefront per slab runs in between and leaves one record per slab, which the consumers read instead.
+constexpr int kNchwMergeInline = 256;
+// forward: (mean, M2) per slab -> out: 2 planes [N * G]
+template <typename A>
+__global__ __launch_bounds__(kBlock) void nchw_stats_compact_kernel(const A *__restrict__ part, A *__restrict__ out, NchwGeo q) {
+  const int64_t item = (int64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+  if (item >= q.N * q.G) return;
+  const int64_t n = item / q.G;
+  A mean, m2;
+  nchw_merge_slab<A>(part, q, n, (int)(item - n * q.G), threadIdx.x & 63, mean, m2);
+  if ((threadIdx.x & 63) == 0) {
+    out[item] = mean;
+    out[q.N * q.G + item] = m2;
+  }
+}
+// The slab's group sums A = sum_c gamma_c S1_c and B = sum_c gamma_c S2_c from its D * chunks partials (64 lanes).
+template <typename A, typename PT>
+__device__ __forceinline__ void nchw_group_sums(const A *__restrict__ part, const void *w, const NchwGeo &q, int64_t n, int g,
+                                                int lane, A &ta, A &tb) {
+  const int64_t plane = q.rows * q.chunks;
+  const int64_t first = (n * q.C + (int64_t)g * q.D) * q.chunks;
+  const int64_t P = (int64_t)q.D * q.chunks;
+  ta = (A)0;
+  tb = (A)0;
+  for (int64_t i = lane; i < P; i += 64) {
+    const int cl = (int)(i / q.chunks);
+    const A gm = w ? load_param<PT, A>(w, g * q.D + cl) : (A)1;
+    ta += gm * part[first + i];
+    tb += gm * part[plane + first + i];
+  }
+  segment_sum2(ta, tb, 64);
+}
+// backward: (A, B) per slab -> out: 2 planes [N * G]
+template <typename A, typename PT>
+__global__ __launch_bounds__(kBlock) void nchw_bwd_compact_kernel(const A *__restrict__ part, const void *w, A *__restrict__ out,
+                                                                  NchwGeo q) {
+  const int64_t item = (int64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+  if (item >= q.N * q.G) return;
+  const int64_t n = item / q.G;
+  A ta, tb;
+  nchw_group_sums<A, PT>(part, w, q, n, (int)(item - n * q.G), threadIdx.x & 63, ta, tb);
+  if ((threadIdx.x & 63) == 0) {
+    out[item] = ta;
+    out[q.N * q.G + item] = tb;
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
-// Forward pass 2: every wavefront merges its slab's partials, then y = act(x * a + b) on its chunk with
+// Forward pass 2: every wavefront merges its slab's partials (or reads the slab's compacted record), then y = act(x * a + b) on its chunk with
 // a = rstd * gamma_c, b = beta_c - mean * a.  The wavefront on the first chunk of a slab reports mean / rstd.
 // ---------------------------------------------------------------------------------------------
 template <typename T, typename PT, int VEC, int ACT>
 __global__ __launch_bounds__(kBlock) void nchw_apply_kernel(const T *__restrict__ x, T *__restrict__ y,
-                                                            const acc_t<T> *__restrict__ part, const void *w, const void *b,
-                                                            void *mean_out, void *rstd_out, int sdtype, acc_t<T> eps, NchwGeo q) {
+                                                            const acc_t<T> *__restrict__ part, const acc_t<T> *__restrict__ compact,
+                                                            const void *w, const void *b, void *mean_out, void *rstd_out,
+                                                            int sdtype, acc_t<T> eps, NchwGeo q) {
   using A = acc_t<T>;
   using LV = LaneVec<T, VEC>;
   NchwPos p;
@@ -148,7 +199,12 @@ __global__ __launch_bounds__(kBlock) void nchw_apply_kernel(const T *__restrict_
   const A gamma = w ? load_param<PT, A>(w, p.c) : (A)1;
   const A beta = b ? load_param<PT, A>(b, p.c) : (A)0;
   A mean, m2;
-  nchw_merge_slab<A>(part, q, p.n, p.g, p.lane, mean, m2);
+  if (compact) {
+    mean = compact[p.n * q.G + p.g];
+    m2 = compact[q.N * q.G + p.n * q.G + p.g];
+  } else {
+    nchw_merge_slab<A>(part, q, p.n, p.g, p.lane, mean, m2);
+  }
   const A rs = fast_rsqrt(m2 * fast_rcp((A)q.D * (A)q.R) + eps);
   if (p.lane == 0 && p.k == 0 && p.c == p.g * q.D) {
     if (mean_out) store_scalar<A>(mean_out, p.n * q.G + p.g, sdtype, mean);
@@ -226,8 +282,8 @@ __global__ __launch_bounds__(kBlock) void nchw_bwd_reduce_kernel(const T *__rest
 template <typename T, typename PT, int VEC, int ACT>
 __global__ __launch_bounds__(kBlock) void nchw_bwd_dx_kernel(const T *__restrict__ x, const T *__restrict__ dy, T *__restrict__ dx,
                                                              const void *mean, const void *rstd, int sdtype, const void *w,
-                                                             const void *b, const acc_t<T> *__restrict__ part, void *dw, void *db,
-                                                             NchwGeo q) {
+                                                             const void *b, const acc_t<T> *__restrict__ part,
+                                                             const acc_t<T> *__restrict__ compact, void *dw, void *db, NchwGeo q) {
   using A = acc_t<T>;
   using LV = LaneVec<T, VEC>;
   NchwPos p;
@@ -267,19 +323,13 @@ __global__ __launch_bounds__(kBlock) void nchw_bwd_dx_kernel(const T *__restrict
       if (db) store_param<PT, A>(db, p.c, t2);
     }
   }
-  // group sums from the slab's D * chunks partials
-  A ta = (A)0, tb = (A)0;
-  {
-    const int64_t plane = q.rows * q.chunks;
-    const int64_t first = (p.n * q.C + (int64_t)p.g * q.D) * q.chunks;
-    const int P = q.D * q.chunks;
-    for (int i = p.lane; i < P; i += 64) {
-      const int cl = i / q.chunks;
-      const A gm = w ? load_param<PT, A>(w, p.g * q.D + cl) : (A)1;
-      ta += gm * part[first + i];
-      tb += gm * part[plane + first + i];
-    }
-    segment_sum2(ta, tb, 64);
+  // group sums from the slab's D * chunks partials (or the slab's compacted record)
+  A ta, tb;
+  if (compact) {
+    ta = compact[p.n * q.G + p.g];
+    tb = compact[q.N * q.G + p.n * q.G + p.g];
+  } else {
+    nchw_group_sums<A, PT>(part, w, q, p.n, p.g, p.lane, ta, tb);
   }
   const A s = fast_rcp((A)q.D * (A)q.R);
   const A c1 = (mu * tb - ta) * s * rs * rs * rs;

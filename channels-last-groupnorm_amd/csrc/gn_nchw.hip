@@ -50,16 +50,29 @@ template <typename PT, int VEC, int ACT> void fwd_launch(const NchwArgs &a, cons
   A *part = (A *)a.ws;
   const unsigned grid = wave_grid(q.rows * q.chunks);
   launch(kKindNchwStats, (nchw_stats_kernel<elem_t, VEC>), dim3(grid), dim3(kBlock), a.stream, (const elem_t *)a.x, part, q);
+  A *compact = nullptr;
+  if ((int64_t)q.D * q.chunks > kNchwMergeInline) {  // many partials per slab: merge each slab once, not once per wavefront
+    compact = part + nchw_partial_elems(a.N, a.C, a.R, VEC, false);
+    launch(kKindNchwStats, (nchw_stats_compact_kernel<A>), dim3(wave_grid(q.N * q.G)), dim3(kBlock), a.stream, (const A *)part,
+           compact, q);
+  }
   launch(kKindNchwApply, (nchw_apply_kernel<elem_t, PT, VEC, ACT>), dim3(grid), dim3(kBlock), a.stream, (const elem_t *)a.x,
-         (elem_t *)a.y, (const A *)part, a.w, a.b, a.mean_out, a.rstd_out, a.sdtype, (A)a.eps, q);
+         (elem_t *)a.y, (const A *)part, (const A *)compact, a.w, a.b, a.mean_out, a.rstd_out, a.sdtype, (A)a.eps, q);
 }
 template <typename PT, int VEC, int ACT> void bwd_launch(const NchwArgs &a, const NchwGeo &q) {
   A *part = (A *)a.ws;
   const unsigned grid = wave_grid(q.rows * q.chunks);
   launch(kKindNchwBwdReduce, (nchw_bwd_reduce_kernel<elem_t, PT, VEC, ACT>), dim3(grid), dim3(kBlock), a.stream,
          (const elem_t *)a.x, (const elem_t *)a.dy, a.mean, a.rstd, a.sdtype, a.w, a.b, part, q);
+  A *compact = nullptr;
+  if ((int64_t)q.D * q.chunks > kNchwMergeInline) {
+    compact = part + nchw_partial_elems(a.N, a.C, a.R, VEC, true);
+    launch(kKindNchwBwdReduce, (nchw_bwd_compact_kernel<A, PT>), dim3(wave_grid(q.N * q.G)), dim3(kBlock), a.stream,
+           (const A *)part, a.w, compact, q);
+  }
   launch(kKindNchwBwdDx, (nchw_bwd_dx_kernel<elem_t, PT, VEC, ACT>), dim3(grid), dim3(kBlock), a.stream, (const elem_t *)a.x,
-         (const elem_t *)a.dy, (elem_t *)a.dx, a.mean, a.rstd, a.sdtype, a.w, a.b, (const A *)part, a.dw, a.db, q);
+         (const elem_t *)a.dy, (elem_t *)a.dx, a.mean, a.rstd, a.sdtype, a.w, a.b, (const A *)part, (const A *)compact, a.dw,
+         a.db, q);
 }
 template <typename PT, int VEC> void dispatch_act(const NchwArgs &a, const NchwGeo &q) {
   switch (a.act) {

@@ -23,6 +23,8 @@ SHAPES = [
     ((4, 1920, 289), 32),   # many short rows
     ((2, 16, 300), 16),     # one channel per group
     ((2, 24, 520), 1),      # one group
+    ((2, 512, 4096), 1),    # one group of many long rows: more partials per slab than a consumer merges itself
+    ((1, 16, 70000), 2),    # the same from few, very long rows (fp32: 8 x 69 partials per slab)
 ]
 
 
