@@ -43,6 +43,9 @@ struct SyncArea {
   unsigned rec_bytes;
   void *crecs;                // backward: 16-byte records {S1, S2, epoch} per (sample, tile, channel) of the whole tensor
   unsigned crec_bytes;
+  void *frecs;                // 16-byte records {value0, value1, epoch} per (sample, group): results of the second level
+  unsigned frec_bytes;        // (two_level != 0 only)
+  int two_level;              // the groups' tile records are merged once, by one workgroup per group, not by every workgroup
   unsigned long long epoch;   // value that marks "written in this call"
   const unsigned long long *generation;  // device counter that replaces the epoch in captured launches (resident_epoch)
   unsigned long long *status; // set to the epoch if a wait of this call timed out
@@ -87,6 +90,9 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t record_buffer(const SyncArea &
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t channel_record_buffer(const SyncArea &s) {
   return __builtin_amdgcn_make_buffer_rsrc(s.crecs, 0, (int)s.crec_bytes, 0x27000);
 }
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t final_record_buffer(const SyncArea &s) {
+  return __builtin_amdgcn_make_buffer_rsrc(s.frecs, 0, (int)s.frec_bytes, 0x27000);
+}
 __device__ __forceinline__ void record_store(__amdgpu_buffer_rsrc_t r, int64_t idx, float v0, float v1,
                                              unsigned long long epoch) {
   const u32x4 rec = {__builtin_bit_cast(unsigned, v0), __builtin_bit_cast(unsigned, v1), (unsigned)epoch,
@@ -120,6 +126,48 @@ __device__ __forceinline__ int record_slot(const PartialGeo &q, int G, int n, in
 
 // What a result is replaced by when a wait expired: not a number, so that the call's output cannot pass for one.
 __device__ __forceinline__ float poison() { return __builtin_nanf(""); }
+// Two-level exchange.  With T row tiles per sample every workgroup polls T records for each group of its chunk: fine for a
+// few dozen tiles, but the polling traffic grows with T squared (512 tiles x 16 groups: 8192 records per workgroup, as many
+// bytes as the tensor itself per round of polls).  Beyond a bound set by the host, each group's tile records are instead
+// merged ONCE, by the workgroup that owns the group -- tile (group index inside the chunk) mod T of the chunk in which
+// the group starts -- with all 256 lanes, and published as one final record per (sample, group) that everybody polls.
+// One more round trip, a few thousand times less traffic.
+__device__ __forceinline__ bool owns_group(const Plan &p, const LanePos &l, int gi) {
+  return (l.g_lo + gi) * p.D >= l.cstart && gi % p.tiles == l.tile;
+}
+// Sum of two values over the 256 lanes of the workgroup (fixed tree: wavefront, then the four wavefronts in order);
+// every lane gets the result.  Uses 8 floats of LDS at `scratch`; the caller's other LDS data is not touched.
+template <typename A> __device__ __forceinline__ void block_sum2(A &a, A &b, A *scratch) {
+  segment_sum2(a, b, 64);
+  __syncthreads();  // scratch may still be read from a previous use
+  if ((threadIdx.x & 63) == 0) {
+    scratch[threadIdx.x >> 6] = a;
+    scratch[4 + (threadIdx.x >> 6)] = b;
+  }
+  __syncthreads();
+  a = (scratch[0] + scratch[1]) + (scratch[2] + scratch[3]);
+  b = (scratch[4] + scratch[5]) + (scratch[6] + scratch[7]);
+}
+// Wait for the final record of (sample, group) slot; false (and NaN values) if the wait expires.
+__device__ __forceinline__ void poll_final(const SyncArea &s, __amdgpu_buffer_rsrc_t fb, int slot, float &v0, float &v1) {
+  int spins = 0;
+  while (true) {
+    const u32x4 rec = record_load(fb, slot);
+    if (record_ready(rec, s.epoch) && s.max_spins != kForcedTimeout) {
+      const unsigned u0 = rec.x, u1 = rec.y;
+      v0 = __builtin_bit_cast(float, u0);
+      v1 = __builtin_bit_cast(float, u1);
+      return;
+    }
+    if (++spins > s.max_spins) {
+      *s.status = s.epoch;
+      v0 = poison();
+      v1 = poison();
+      return;
+    }
+    __builtin_amdgcn_s_sleep(2);
+  }
+}
 // Collect the records of group g (all tiles of the chunks that hold a piece of it) with L lanes: each lane polls its
 // own records until they carry this call's epoch, kRecFast at a time (they stay in registers: the round trip that
 // finds them ready also brings their values), and hands (value0, value1, count) of each to body.  If a wait expires,
@@ -326,7 +374,50 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
     record_store(rb, record_slot(q, p.G, (int)n, l.tile, l.chunk, g), mu, s2, sync.epoch);
   });
   trace_point(sync, 2);
-  {
+  if (sync.two_level) {
+    // second level: the groups this workgroup owns, one at a time with all 256 lanes (usually one group or none)
+    const __amdgpu_buffer_rsrc_t fb = final_record_buffer(sync);
+    const A total = (A)p.D * (A)p.R;
+    __shared__ A sm_x[12];
+    for (int gi = l.tile; gi < l.ng; gi += p.tiles) {  // uniform over the workgroup
+      if (!owns_group(p, l, gi)) continue;
+      const int g = l.g_lo + gi;
+      A nl = (A)0, kl = (A)0, s1 = (A)0, s2 = (A)0;
+      for_group_records(sync, rb, q, p, n, g, true, kBlock, threadIdx.x, [&](float mu, float mm, float cnt) {
+        if (nl == (A)0) kl = mu;
+        const A d = mu - kl;
+        nl += cnt;
+        s1 += cnt * d;
+        s2 += mm + cnt * d * d;
+      });
+      const A inv = nl > (A)0 ? fast_rcp(nl) : (A)0;
+      const A mean_l = kl + s1 * inv;
+      const A m2_l = s2 - s1 * s1 * inv;
+      __syncthreads();
+      if (threadIdx.x == 0) sm_x[8] = mean_l;  // lane 0 always has a record: the pivot of the merge across lanes
+      __syncthreads();
+      const A K = sm_x[8];
+      const A d = nl > (A)0 ? mean_l - K : (A)0;
+      A t1 = nl * d, t2 = m2_l + nl * d * d;
+      block_sum2(t1, t2, sm_x);
+      if (threadIdx.x == 0) {
+        const A dm = t1 * fast_rcp(total);
+        const A gmean = K + dm;
+        const A rs = fast_rsqrt((t2 - t1 * dm) * fast_rcp(total) + eps);
+        record_store(fb, (int)n * p.G + g, gmean, rs, sync.epoch);
+        if (mean_out) store_scalar<A>(mean_out, n * p.G + g, sdtype, gmean);
+        if (rstd_out) store_scalar<A>(rstd_out, n * p.G + g, sdtype, rs);
+      }
+    }
+    // everybody: one final record per group of the chunk
+    for (int gi = threadIdx.x; gi < l.ng; gi += kBlock) {
+      float gmean, rs;
+      poll_final(sync, fb, (int)n * p.G + l.g_lo + gi, gmean, rs);
+      sm0[gi] = gmean;
+      sm1[gi] = rs;
+    }
+    __syncthreads();
+  } else {
     // merge the records of the chunk's groups (exact two-pass form, compute_stats_pt2's job:
     // src/gnnhwc/csrc/gn_kernel.cu:226-292); rstd = 1 / sqrt(M2 / n + eps)
     const int L = merge_lanes(q, p.D);
@@ -531,7 +622,34 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
   }
   __syncthreads();
   trace_point(sync, 2);
-  {
+  if (sync.two_level) {
+    // second level (see owns_group): the groups this workgroup owns, one at a time with all 256 lanes
+    const __amdgpu_buffer_rsrc_t fb = final_record_buffer(sync);
+    __shared__ A sm_x[8];
+    for (int gi = l.tile; gi < l.ng; gi += p.tiles) {  // uniform over the workgroup
+      if (!owns_group(p, l, gi)) continue;
+      const int g = l.g_lo + gi;
+      A ta = (A)0, tb = (A)0;
+      for_group_records(sync, rb, q, p, n, g, true, kBlock, threadIdx.x, [&](float ra, float rbv, float) {
+        ta += ra;
+        tb += rbv;
+      });
+      block_sum2(ta, tb, sm_x);
+      if (threadIdx.x == 0) {
+        const A mu = sm_mu[gi];
+        const A rs = sm_rs[gi];
+        const A s = fast_rcp((A)p.D * (A)p.R);
+        const A k1 = (mu * tb - ta) * s * rs * rs * rs;
+        record_store(fb, (int)n * p.G + g, k1, -mu * k1 - tb * s * rs, sync.epoch);
+      }
+    }
+    for (int gi = threadIdx.x; gi < l.ng; gi += kBlock) {
+      float k1, k2;
+      poll_final(sync, fb, (int)n * p.G + l.g_lo + gi, k1, k2);
+      sm1[gi] = k1;
+      sm2[gi] = k2;
+    }
+  } else {
     const int L = merge_lanes(q, p.D);
     const int nseg = kBlock >> __builtin_ctz(L);  // L is a power of two
     const int seg = threadIdx.x >> __builtin_ctz(L), sl = threadIdx.x & (L - 1);

@@ -105,7 +105,19 @@ constexpr size_t kWorkspaceHeader = 256;
 // The resident kernels keep their partial results and one flag per workgroup in the same workspace.
 constexpr int kMaxResidentBlocks = 4 * kNumCU;
 inline size_t resident_rec_bytes(int64_t G) { return (size_t)16 * G * kMaxResidentBlocks; }
-inline size_t resident_fwd_bytes(int64_t G) { return kWorkspaceHeader + align_up(resident_rec_bytes(G), 256); }
+// Final records of the two-level exchange, one per (sample, group) of a launch: a launch has at most kMaxResidentBlocks samples.
+inline size_t resident_frec_bytes(int64_t G) { return (size_t)16 * G * kMaxResidentBlocks; }
+inline size_t resident_fwd_bytes(int64_t G) {
+  return kWorkspaceHeader + align_up(resident_rec_bytes(G), 256) + align_up(resident_frec_bytes(G), 256);
+}
+// All-to-all or two-level exchange: records a workgroup would poll in the all-to-all form (tiles x chunks per group x
+// groups per chunk); beyond this bound the polling traffic of the whole launch rivals the tensor itself.
+constexpr int kTwoLevelRecords = 1024;
+inline bool two_level_exchange(const Plan &p) {
+  const int chunk_channels = p.lpr * p.vec;
+  const int64_t per_group = (int64_t)p.tiles * ((p.D - 1) / chunk_channels + 2);
+  return per_group * p.gmax > kTwoLevelRecords && p.tiles > 1;
+}
 // chunk_channels = channels per workgroup (lpr * vec): N * tiles * C = workgroups * chunk_channels
 // A tensor of several samples that is too large for one single-launch kernel may still be run as up to
 // kMaxBatches such launches over consecutive groups of samples (samples share nothing but dgamma / dbeta).
@@ -118,7 +130,8 @@ inline size_t resident_crec_bytes(int64_t chunk_channels) {
   return align_up(one > many ? one : many, 256);
 }
 inline size_t resident_bwd_bytes(int64_t chunk_channels, int64_t G) {
-  return kWorkspaceHeader + resident_crec_bytes(chunk_channels) + align_up(resident_rec_bytes(G), 256);
+  return kWorkspaceHeader + resident_crec_bytes(chunk_channels) + align_up(resident_rec_bytes(G), 256) +
+         align_up(resident_frec_bytes(G), 256);
 }
 // A fresh nonzero 64-bit value per call (gn_api.hip).
 unsigned long long next_epoch();

@@ -115,6 +115,9 @@ ResidentWorkspace resident_fwd_ws(void *ws, const Plan &p) {
   char *base = (char *)ws + kWorkspaceHeader;
   r.sync.recs = base;
   r.sync.rec_bytes = (unsigned)resident_rec_bytes(p.G);
+  r.sync.frecs = base + align_up(resident_rec_bytes(p.G), 256);
+  r.sync.frec_bytes = (unsigned)resident_frec_bytes(p.G);
+  r.sync.two_level = two_level_exchange(p) ? 1 : 0;
   r.sync.crecs = nullptr;
   r.sync.crec_bytes = 0;
   r.sync.status = resident_status();
@@ -133,6 +136,9 @@ ResidentWorkspace resident_bwd_ws(void *ws, const Plan &p) {
   r.sync.crec_bytes = (unsigned)resident_crec_bytes(cc);
   r.sync.recs = base + resident_crec_bytes(cc);
   r.sync.rec_bytes = (unsigned)resident_rec_bytes(p.G);
+  r.sync.frecs = base + resident_crec_bytes(cc) + align_up(resident_rec_bytes(p.G), 256);
+  r.sync.frec_bytes = (unsigned)resident_frec_bytes(p.G);
+  r.sync.two_level = two_level_exchange(p) ? 1 : 0;
   r.sync.status = resident_status();
   r.sync.generation = nullptr;
   r.sync.max_spins = resident_spin_limit();
