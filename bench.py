@@ -340,7 +340,7 @@ def timeline(names, device, reps=5):
                 torch.cuda.synchronize()
                 _cabi.check(_cabi.lib.gnnhwc_debug_read_trace(words.ctypes.data, words.size), "gnnhwc_debug_read_trace")
                 t = words.astype(np.int64)
-                live = t[:, 0] >= t[:, 0].max() - 5000  # within 50 us of the latest start: this launch
+                live = t[:, 0] >= t[:, 0].max() - 300  # started within 3 us of the latest start: the workgroups of this launch
                 t = t[live]
                 rel = (t - t[:, 0].min()) / 100.0
                 taken = {}
