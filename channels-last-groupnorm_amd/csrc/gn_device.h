@@ -339,6 +339,13 @@ template <typename A> __device__ __forceinline__ void segment_sum2(A &a, A &b, i
     b += ob;
   }
 }
+// Segment index of a thread when the workgroup is cut into segments of L lanes (a power of two <= 64), numbered so that
+// consecutive segments sit in DIFFERENT wavefronts: the first few groups of a chunk then keep all four SIMDs of the CU
+// busy instead of queueing in the first wavefront.
+__device__ __forceinline__ int spread_segment(int L) {
+  const int wave = threadIdx.x >> 6, sub = (threadIdx.x & 63) >> __builtin_ctz(L);
+  return sub * (kBlock / 64) + wave;
+}
 __device__ __forceinline__ int pow2_ceil_clamped(int v, int hi) {
   int p = 1;
   while (p < v && p < hi) p <<= 1;

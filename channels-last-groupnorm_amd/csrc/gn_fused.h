@@ -607,7 +607,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
   {
     const int L = pow2_ceil_clamped(p.D < l.wch ? p.D : l.wch, 64);
     const int nseg = kBlock >> __builtin_ctz(L);  // L is a power of two
-    const int seg = threadIdx.x >> __builtin_ctz(L), sl = threadIdx.x & (L - 1);
+    const int seg = spread_segment(L), sl = threadIdx.x & (L - 1);
     for (int base = 0; base < l.ng; base += nseg) {
       const int gi = base + seg;
       const int g = l.g_lo + gi;

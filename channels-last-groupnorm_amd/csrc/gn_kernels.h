@@ -360,7 +360,7 @@ __device__ __forceinline__ void block_group_moments(const Plan &p, const LanePos
   const int nc_max = p.D < l.wch ? p.D : l.wch;
   const int L = pow2_ceil_clamped(nc_max, 16);  // lanes per group: a DPP row at most
   const int nseg = kBlock >> __builtin_ctz(L);  // L is a power of two
-  const int seg = threadIdx.x >> __builtin_ctz(L), sl = threadIdx.x & (L - 1);
+  const int seg = spread_segment(L), sl = threadIdx.x & (L - 1);
   const A nrows = (A)l.len;
   for (int base = 0; base < l.ng; base += nseg) {
     const int gi = base + seg;
