@@ -52,6 +52,9 @@ def parse_args():
     ap.add_argument("--fused-add", action="store_true",
                     help="also time gnnhwc_fwd_add (residual + sum output fused into the forward) against an elementwise "
                          "addition followed by gnnhwc_fwd, per shape (reported under 'fused_add')")
+    ap.add_argument("--cast", action="store_true",
+                    help="also time gnnhwc_fwd_cast (float32 x, y written as bfloat16 by the kernel) against gnnhwc_fwd followed "
+                         "by a cast kernel, on the float32 versions of the workload's shapes (reported under 'cast')")
     ap.add_argument("--nchw", action="store_true",
                     help="also time the channels-first entry points on the same shapes against torch's GroupNorm + activation "
                          "on channels-first tensors (reported under 'channels_first')")
@@ -485,6 +488,48 @@ def fused_add_table(names, device, steps, warmup):
     return out
 
 
+def cast_table(names, device, steps, warmup):
+    """Forward of float32 data with y leaving as bfloat16 (reads S, writes S / 2) against the sequence a caller of the
+    plain forward runs for a half-precision consumer: gnnhwc_fwd (2 S) and a cast kernel (1.5 S more)."""
+    import torch
+    import workloads as configs
+
+    out = {}
+    for n in names:
+        cfg = configs.CONFIGS[n]._replace(dtype="fp32")
+        p = Problem(cfg, device)
+        b = p.sets[0]
+        x = b["x"]
+        y16 = torch.empty(x.shape, dtype=torch.bfloat16, device=device)
+        stream_of = lambda: torch.cuda.current_stream().cuda_stream  # noqa: E731
+
+        def fused():
+            rc = p.lib.gnnhwc_fwd_cast(x.data_ptr(), p.w.data_ptr(), p.b.data_ptr(), y16.data_ptr(), p.mean.data_ptr(),
+                                       p.rstd.data_ptr(), p.N, p.R, p.C, p.G, 1e-5, p.act, p.dt, p.dt, p.sdt, 3,
+                                       p.ws_f.data_ptr(), p.ws_f.numel(), stream_of())
+            if rc != 0:
+                raise RuntimeError(p.lib.gnnhwc_last_error().decode())
+
+        def unfused():
+            rc = p.lib.gnnhwc_fwd(x.data_ptr(), p.w.data_ptr(), p.b.data_ptr(), b["y"].data_ptr(), p.mean.data_ptr(),
+                                  p.rstd.data_ptr(), p.N, p.R, p.C, p.G, 1e-5, p.act, p.dt, p.dt, p.sdt,
+                                  p.ws_f.data_ptr(), p.ws_f.numel(), stream_of())
+            if rc != 0:
+                raise RuntimeError(p.lib.gnnhwc_last_error().decode())
+            y16.copy_(b["y"])
+
+        r = {}
+        for key, fn in (("fused", fused), ("unfused", unfused)):
+            t = min(time_region(fn, steps, warmup, False) for _ in range(3)) / steps
+            r[key + "_us"] = round(t * 1e6, 3)
+            r[key + "_gbps"] = round(1.5 * p.S / t / 1e9, 1)  # algorithmic bytes of the FUSED form / time
+        r["speedup"] = round(r["unfused_us"] / r["fused_us"], 3)
+        out[n + "_fp32"] = r
+        del p
+        torch.cuda.empty_cache()
+    return out
+
+
 def nchw_table(names, device, steps, warmup):
     """gnnhwc_fwd_nchw / gnnhwc_bwd_nchw (two launches forward, three backward; algorithmic bytes 2 S / 3 S as for the
     channels-last path) against what the reference does with channels-first input: torch's GroupNorm followed by the
@@ -696,6 +741,8 @@ def main():
     }
     if args.nchw:
         line["channels_first"] = nchw_table(head_names, device, max(20, args.steps // 2), args.warmup)
+    if args.cast:
+        line["cast"] = cast_table(head_names, device, max(20, args.steps // 2), args.warmup)
     if args.fused_add:
         line["fused_add"] = fused_add_table(head_names, device, max(20, args.steps // 2), args.warmup)
     if not args.no_cpu_baseline:

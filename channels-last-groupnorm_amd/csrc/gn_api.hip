@@ -481,17 +481,23 @@ size_t gnnhwc_bwd_workspace_bytes(int64_t N, int64_t R, int64_t C, int64_t G, in
 
 static int forward(const void *x, const AddArgs &add, const void *weight, const void *bias, void *y, void *mean, void *rstd,
                    int64_t N, int64_t R, int64_t C, int64_t G, double eps, int act, int dtype, int param_dtype,
-                   int stats_dtype, void *workspace, size_t workspace_bytes, void *stream, bool streaming_only = false) {
+                   int stats_dtype, void *workspace, size_t workspace_bytes, void *stream, bool streaming_only = false,
+                   int y_dtype = -1) {
   int rc = check_shape(N, R, C, G, dtype);
   if (rc != GNNHWC_OK) return rc;
   rc = check_dtypes(dtype, param_dtype, stats_dtype);
   if (rc != GNNHWC_OK) return rc;
   if (act < GN_ACT_IDENTITY || act > GN_ACT_GELU_TANH)
     return fail(GNNHWC_ERR_INVALID_ARGUMENT, "unknown activation code %d", act);
+  if (y_dtype < 0) y_dtype = dtype;
+  if (y_dtype != dtype && !(dtype == GN_F32 && (y_dtype == GN_F16 || y_dtype == GN_BF16)))
+    return fail(GNNHWC_ERR_INVALID_ARGUMENT, "y_dtype %d with dtype %d: y is written in dtype, or as F16 / BF16 for F32 data",
+                y_dtype, dtype);
   if (N == 0 || R == 0) return GNNHWC_OK;  // nothing to normalise; mean / rstd of an empty slab are left untouched
   rc = check_resident_health();
   if (rc != GNNHWC_OK) return rc;
   if (!x || !y) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "x and y must not be null");
+  if (y_dtype != dtype && y == x) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "y of another type than x cannot replace x in place");
   const size_t need = streaming_only ? align_up(fwd_ws_bytes(N, R, C, G, dtype, true), 256) : gnnhwc_fwd_workspace_bytes(N, R, C, G, dtype);
   if (!workspace || !aligned16(workspace) || workspace_bytes < need)
     return fail(GNNHWC_ERR_WORKSPACE, "forward workspace must be 16-byte aligned and at least %zu bytes (got %p, %zu bytes)",
@@ -502,7 +508,7 @@ static int forward(const void *x, const AddArgs &add, const void *weight, const 
   a.streaming_only = streaming_only;
   a.add = add;
   a.x = x; a.w = weight; a.b = bias; a.y = y; a.mean = mean; a.rstd = rstd;
-  a.eps = eps; a.act = act; a.pdtype = param_dtype; a.sdtype = stats_dtype;
+  a.eps = eps; a.act = act; a.pdtype = param_dtype; a.sdtype = stats_dtype; a.ydtype = y_dtype;
   a.ws = workspace; a.stream = (hipStream_t)stream;
   a.plan = make_plan(N, R, C, G, vector_ok ? vec : 1, 1);
   if (a.plan.nchunk > 65535) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "too many channels for this build (C = %lld)", (long long)C);
@@ -523,6 +529,15 @@ int gnnhwc_fwd(const void *x, const void *weight, const void *bias, void *y, voi
   const AddArgs none = {nullptr, nullptr, GN_F32, nullptr};
   return forward(x, none, weight, bias, y, mean, rstd, N, R, C, G, eps, act, dtype, param_dtype, stats_dtype, workspace,
                  workspace_bytes, stream);
+}
+
+int gnnhwc_fwd_cast(const void *x, const void *weight, const void *bias, void *y, void *mean, void *rstd, int64_t N,
+                    int64_t R, int64_t C, int64_t G, double eps, int act, int dtype, int param_dtype, int stats_dtype,
+                    int y_dtype, void *workspace, size_t workspace_bytes, void *stream) {
+  if (y_dtype < GN_F32 || y_dtype > GN_BF16) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "unknown y_dtype code %d", y_dtype);
+  const AddArgs none = {nullptr, nullptr, GN_F32, nullptr};
+  return forward(x, none, weight, bias, y, mean, rstd, N, R, C, G, eps, act, dtype, param_dtype, stats_dtype, workspace,
+                 workspace_bytes, stream, false, y_dtype);
 }
 
 size_t gnnhwc_fwd_static_scratch_bytes(int64_t N, int64_t R, int64_t C, int64_t G, int dtype) {

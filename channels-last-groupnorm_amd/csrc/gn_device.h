@@ -29,6 +29,7 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ float bf16_bits_to_float(uint32_t hi16_in_place) {
@@ -144,6 +145,35 @@ template <typename LV, typename T> __device__ __forceinline__ void store_streami
 }
 template <typename LV, typename T> __device__ __forceinline__ typename LV::raw_t load_streaming(const T *p) {
   return __builtin_nontemporal_load((const typename LV::raw_t *)p);
+}
+// One lane vector of forward results, stored at element `e` of y.  y normally has the data type; float data may also be
+// written as a 16-bit type (ydtype GN_F16 / GN_BF16; the host admits nothing else), each value rounded once from the
+// fp32 result: the layer that consumes y in half precision then reads half the bytes and no cast kernel runs between.
+template <typename T, int VEC, typename A>
+__device__ __forceinline__ void store_result(T *y, int64_t e, const A (&v)[VEC], int ydtype) {
+  using LV = LaneVec<T, VEC>;
+  if constexpr (sizeof(T) == 4) {
+    if (ydtype != GN_F32) {
+      uint16_t *yp = (uint16_t *)y + e;
+      if constexpr (VEC == 4) {
+        u32x2 r;
+        if (ydtype == GN_BF16) {
+          r.x = pack_bf16x2(v[0], v[1]);
+          r.y = pack_bf16x2(v[2], v[3]);
+        } else {
+          const f16x2 lo = {(_Float16)v[0], (_Float16)v[1]}, hi = {(_Float16)v[2], (_Float16)v[3]};
+          r.x = __builtin_bit_cast(uint32_t, lo);
+          r.y = __builtin_bit_cast(uint32_t, hi);
+        }
+        __builtin_nontemporal_store(r, (u32x2 *)yp);
+      } else {
+        const _Float16 h = (_Float16)v[0];
+        *yp = ydtype == GN_BF16 ? float_to_bf16_bits(v[0]) : __builtin_bit_cast(uint16_t, h);
+      }
+      return;
+    }
+  }
+  store_streaming<LV>(y + e, LV::pack(v));
 }
 
 // ---- runtime-typed scalar access to parameters / statistics (read once per workgroup) ----

@@ -238,7 +238,7 @@ constexpr int fused_fwd_waves(int nv, int add) {
 template <typename T, typename PT, int VEC, int ACT, int NV, int ADD>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fwd_waves(NV, ADD)))) void fused_fwd_kernel(
     const T *__restrict__ x, T *__restrict__ y, SyncArea sync_arg, const void *w, const void *b, void *mean_out,
-    void *rstd_out, int sdtype, acc_t<T> eps, AddArgs add, Plan p) {
+    void *rstd_out, int sdtype, int ydtype, acc_t<T> eps, AddArgs add, Plan p) {
   using A = acc_t<T>;
   using LV = LaneVec<T, VEC>;
   const SyncArea sync = resident_epoch(sync_arg);
@@ -472,7 +472,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
         LV::unpack(buf[u], v);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) v[j] = act_fwd<ACT, A>(v[j] * sa[j] + sb[j]);
-        store_streaming<LV>(y + off + (int64_t)u * step, LV::pack(v));
+        store_result<T, VEC>(y, off + (int64_t)u * step, v, ydtype);
       }
     }
   }

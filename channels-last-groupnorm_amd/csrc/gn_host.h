@@ -37,6 +37,7 @@ struct FwdArgs {
   void *y, *mean, *rstd;
   double eps;
   int act, pdtype, sdtype;
+  int ydtype;  // type y is stored in: the data type, or for float data GN_F16 / GN_BF16
   void *ws;
   hipStream_t stream;
   Plan plan;

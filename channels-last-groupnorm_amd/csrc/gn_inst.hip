@@ -52,7 +52,7 @@ dim3 tile_grid(const Plan &p, int extra_x) {
 template <typename PT, int VEC, int ACT> void launch_apply(const FwdArgs &a, const A *part, const PartialGeo &q) {
   const Plan &p = a.plan;
   launch(kKindFwdApply, (apply_kernel<elem_t, PT, VEC, ACT>), tile_grid(p, 0), dim3(kBlock), a.stream, (const elem_t *)a.x,
-         (elem_t *)a.y, part, q, a.w, a.b, a.mean, a.rstd, a.sdtype, (A)a.eps, p);
+         (elem_t *)a.y, part, q, a.w, a.b, a.mean, a.rstd, a.sdtype, a.ydtype, (A)a.eps, p);
 }
 template <typename PT, int VEC> void launch_apply_act(const FwdArgs &a, const A *part, const PartialGeo &q) {
   switch (a.act) {
@@ -187,9 +187,9 @@ template <typename PT, int ACT, int NV, int ADD> bool try_resident_fwd_nv(const 
     if (add.sum_out) add.sum_out = (elem_t *)add.sum_out + n0 * sample;
     if (add.channel_bias) add.channel_bias = (const char *)add.channel_bias + n0 * a.plan.C * stat_size(add.channel_bias_dtype);
     launch(ADD != kAddNone ? kKindFusedFwdAdd : kKindFusedFwd, kernel, tile_grid(pb, 0), dim3(kBlock), a.stream,
-           (const elem_t *)a.x + n0 * sample, (elem_t *)a.y + n0 * sample, r.sync, a.w, a.b,
+           (const elem_t *)a.x + n0 * sample, (elem_t *)((char *)a.y + n0 * sample * stat_size(a.ydtype)), r.sync, a.w, a.b,
            a.mean ? (char *)a.mean + n0 * a.plan.G * stat_size(a.sdtype) : nullptr,
-           a.rstd ? (char *)a.rstd + n0 * a.plan.G * stat_size(a.sdtype) : nullptr, a.sdtype, (A)a.eps, add, pb);
+           a.rstd ? (char *)a.rstd + n0 * a.plan.G * stat_size(a.sdtype) : nullptr, a.sdtype, a.ydtype, (A)a.eps, add, pb);
   }
   return true;
 }

@@ -699,7 +699,7 @@ __device__ __forceinline__ void lane_coeffs(const Plan &p, const LanePos &l, con
 template <typename T, typename PT, int VEC, int ACT>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) void apply_kernel(
     const T *__restrict__ x, T *__restrict__ y, const acc_t<T> *__restrict__ part, PartialGeo q, const void *w,
-    const void *b, void *mean_out, void *rstd_out, int sdtype, acc_t<T> eps, Plan p) {
+    const void *b, void *mean_out, void *rstd_out, int sdtype, int ydtype, acc_t<T> eps, Plan p) {
   using A = acc_t<T>;
   using LV = LaneVec<T, VEC>;
   constexpr int U = kUnrollFwd;
@@ -731,7 +731,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
         else LV::unpack(buf1[u], v);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) v[j] = act_fwd<ACT, A>(v[j] * sa[j] + sb[j]);
-        if (bi * U + u < rows) store_streaming<LV>(y + off + (int64_t)(bi * U + u) * step, LV::pack(v));
+        if (bi * U + u < rows) store_result<T, VEC>(y, off + (int64_t)(bi * U + u) * step, v, ydtype);
       }
     };
     // order of issue: the few small loads the prologue depends on first, then the first batch of x, so that

@@ -21,6 +21,7 @@ SYMBOLS = (
     "gnnhwc_fwd_workspace_bytes",
     "gnnhwc_bwd_workspace_bytes",
     "gnnhwc_fwd",
+    "gnnhwc_fwd_cast",
     "gnnhwc_fwd_add",
     "gnnhwc_fwd_static",
     "gnnhwc_fwd_static_scratch_bytes",
@@ -57,6 +58,8 @@ def _load():
     lib.gnnhwc_bwd_workspace_bytes.restype = sz
     lib.gnnhwc_fwd.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, dbl, ci, ci, ci, ci, vp, sz, vp]
     lib.gnnhwc_fwd.restype = ci
+    lib.gnnhwc_fwd_cast.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, dbl, ci, ci, ci, ci, ci, vp, sz, vp]
+    lib.gnnhwc_fwd_cast.restype = ci
     lib.gnnhwc_fwd_add.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, dbl, ci, ci, ci, ci, ci, vp, sz, vp]
     lib.gnnhwc_fwd_add.restype = ci
     lib.gnnhwc_fwd_static.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, dbl, ci, ci, ci, ci, vp]

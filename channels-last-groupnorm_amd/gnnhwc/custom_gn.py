@@ -136,14 +136,30 @@ def _workspace(nbytes, device, stream_ptr):
 
 def gn_nhwc_fwd(X, weight, bias, G, eps, act_fn_option):
     """gnop::fwd -- custom_gn.cpp:10-42.  X: (N, C, R) channels-last view.  Returns (Y, means, rstds)."""
+    return _nhwc_fwd(X, weight, bias, G, eps, act_fn_option, None, "gnop::fwd")
+
+
+def gn_nhwc_fwd_cast(X, weight, bias, G, eps, act_fn_option, out_dtype):
+    """gnop::fwd_cast (no counterpart in the reference, whose Y has X's dtype, custom_gn.cpp:28): gnop::fwd on float32
+    data with Y written as float16 / bfloat16 by the kernel itself, for a consumer that runs in half precision."""
+    return _nhwc_fwd(X, weight, bias, G, eps, act_fn_option, out_dtype, "gnop::fwd_cast")
+
+
+def _nhwc_fwd(X, weight, bias, G, eps, act_fn_option, out_dtype, opname):
     _check_device(X, "X")
     if X.dim() != 3:
-        raise RuntimeError("gnop::fwd expects X of shape (N, C, R), got %s" % (tuple(X.shape),))
+        raise RuntimeError("%s expects X of shape (N, C, R), got %s" % (opname, tuple(X.shape)))
     N, C, R = X.shape
     dt = _dtype_code(X, "X")
     pdt, w_ptr, b_ptr, _keep = _param_args(weight, bias, C, dt)
     X_nrc = _as_nrc(X)
-    Y = torch.empty_like(X_nrc)
+    if out_dtype is None or out_dtype == X.dtype:
+        Y = torch.empty_like(X_nrc)
+    elif X.dtype == torch.float32 and out_dtype in (torch.float16, torch.bfloat16):
+        Y = torch.empty(X_nrc.shape, dtype=out_dtype, device=X.device)
+    else:
+        raise RuntimeError("%s: out_dtype %s with %s data (float32 data may leave as float16 or bfloat16)"
+                           % (opname, out_dtype, X.dtype))
     sdtype = _stats_dtype(X.dtype)
     means = torch.empty((N, G), dtype=sdtype, device=X.device)
     rstds = torch.empty((N, G), dtype=sdtype, device=X.device)
@@ -151,15 +167,15 @@ def gn_nhwc_fwd(X, weight, bias, G, eps, act_fn_option):
     with _on_device(X.device):
         nbytes = lib.gnnhwc_fwd_workspace_bytes(N, R, C, G, dt)
         if nbytes == 0:
-            raise RuntimeError("gnop::fwd: " + _cabi.last_error())
+            raise RuntimeError(opname + ": " + _cabi.last_error())
         stream = _current_stream_ptr(X.device)
         ws = _workspace(nbytes, X.device, stream)
-        rc = lib.gnnhwc_fwd(
+        rc = lib.gnnhwc_fwd_cast(
             X_nrc.data_ptr(), w_ptr, b_ptr,
             Y.data_ptr(), means.data_ptr(), rstds.data_ptr(),
-            N, R, C, G, float(eps), int(act_fn_option), dt, pdt, _DTYPE_CODE[sdtype],
+            N, R, C, G, float(eps), int(act_fn_option), dt, pdt, _DTYPE_CODE[sdtype], _DTYPE_CODE[Y.dtype],
             ws.data_ptr(), ws.numel(), stream)
-    _cabi.check(rc, "gnop::fwd")
+    _cabi.check(rc, opname)
     return Y.permute(0, 2, 1), means, rstds
 
 
@@ -335,12 +351,15 @@ _op_lib.define("bwd(Tensor dy, Tensor X, Tensor weight, Tensor bias, Tensor mean
                "int act_fn_option) -> (Tensor, Tensor, Tensor)")
 _op_lib.define("fwd_add(Tensor X, Tensor? residual, Tensor? channel_bias, Tensor weight, Tensor bias, int G, float eps, "
                "int act_fn_option, bool return_sum) -> (Tensor, Tensor, Tensor, Tensor)")
+_op_lib.define("fwd_cast(Tensor X, Tensor? weight, Tensor? bias, int G, float eps, int act_fn_option, ScalarType out_dtype) -> "
+               "(Tensor, Tensor, Tensor)")
 _op_lib.define("fwd_nchw(Tensor X, Tensor weight, Tensor bias, int G, float eps, int act_fn_option) -> (Tensor, Tensor, Tensor)")
 _op_lib.define("bwd_nchw(Tensor dy, Tensor X, Tensor weight, Tensor bias, Tensor means, Tensor rstds, int G, "
                "int act_fn_option) -> (Tensor, Tensor, Tensor)")
 _op_lib.impl("fwd_nchw", gn_nchw_fwd, "CompositeExplicitAutograd")
 _op_lib.impl("bwd_nchw", gn_nchw_bwd, "CompositeExplicitAutograd")
 _op_lib.impl("fwd", gn_nhwc_fwd, "CompositeExplicitAutograd")
+_op_lib.impl("fwd_cast", gn_nhwc_fwd_cast, "CompositeExplicitAutograd")
 _op_lib.impl("fwd_add", gn_nhwc_fwd_add, "CompositeExplicitAutograd")
 _op_lib.impl("bwd", gn_nhwc_bwd, "CompositeExplicitAutograd")
 
@@ -412,6 +431,39 @@ def _fwd_backward(ctx, dY, _dmeans, _drstds):
 torch.library.register_autograd("gnop::fwd", _fwd_backward, setup_context=_fwd_setup_context, lib=_op_lib)
 
 
+def _fwd_cast_meta(X, weight, bias, G, eps, act_fn_option, out_dtype):
+    N, C, R = X.shape
+    Y = torch.empty((N, R, C), dtype=out_dtype, device=X.device).permute(0, 2, 1)
+    sdtype = _stats_dtype(X.dtype)
+    return Y, torch.empty((N, G), dtype=sdtype, device=X.device), torch.empty((N, G), dtype=sdtype, device=X.device)
+
+
+_op_lib.impl("fwd_cast", _fwd_cast_meta, "Meta")
+
+
+def _fwd_cast_setup_context(ctx, inputs, output):
+    X, weight, bias, G, _eps, act_fn_option, _out_dtype = inputs
+    _Y, means, rstds = output
+    ctx.save_for_backward(X, weight, bias, means, rstds)
+    ctx.G = G
+    ctx.act_fn_option = act_fn_option
+    ctx.mark_non_differentiable(means, rstds)
+
+
+def _fwd_cast_backward(ctx, dY, _dmeans, _drstds):
+    """The backward kernels have one element type: the 16-bit gradient of Y is widened to X's float32 first."""
+    X, weight, bias, means, rstds = ctx.saved_tensors
+    dY = dY.permute(0, 2, 1).to(X.dtype).contiguous().permute(0, 2, 1)
+    if weight is None:
+        dX, _dw, _db = gn_nhwc_bwd(dY, X, None, None, means, rstds, ctx.G, ctx.act_fn_option)
+        return dX, None, None, None, None, None, None
+    dX, dweight, dbias = torch.ops.gnop.bwd(dY, X, weight, bias, means, rstds, ctx.G, ctx.act_fn_option)
+    return dX, dweight, dbias, None, None, None, None
+
+
+torch.library.register_autograd("gnop::fwd_cast", _fwd_cast_backward, setup_context=_fwd_cast_setup_context, lib=_op_lib)
+
+
 def _fwd_nchw_backward(ctx, dY, _dmeans, _drstds):
     X, weight, bias, means, rstds = ctx.saved_tensors
     dX, dweight, dbias = torch.ops.gnop.bwd_nchw(dY.contiguous(), X, weight, bias, means, rstds, ctx.G, ctx.act_fn_option)
@@ -459,7 +511,7 @@ torch.library.register_autograd("gnop::fwd_add", _fwd_add_backward, setup_contex
 
 
 def group_norm_nhwc(x, weight, bias, num_groups, eps=1e-5, activation="identity", residual=None, channel_bias=None,
-                    return_sum=False):
+                    return_sum=False, out_dtype=None):
     """Functional, traceable form of GN_NHWC.forward for channels-last input (x.stride(1) == 1): the same operator
     and results, differentiated through the operator's registered autograd formula instead of GN_NHWC_Func, so
     torch.compile can keep it in one graph.  weight / bias must be given (use ones / zeros for a non-affine norm).
@@ -467,7 +519,11 @@ def group_norm_nhwc(x, weight, bias, num_groups, eps=1e-5, activation="identity"
     Optional fused additions (no counterpart in the reference): the normalised tensor becomes
     s = x + residual + channel_bias[:, :, None, ...] (residual: x's shape; channel_bias: (N, C), e.g. a time
     embedding), computed inside the kernel and rounded to x's dtype once; with return_sum=True the call returns
-    (y, s) so that s can serve as the next skip connection."""
+    (y, s) so that s can serve as the next skip connection.
+
+    out_dtype (no counterpart in the reference either): float32 input may leave as torch.float16 / torch.bfloat16,
+    written in that type by the kernel (for a convolution that runs in half precision on a float32 residual stream);
+    weight / bias may then be None.  Not combined with the fused additions."""
     if x.stride(1) != 1:
         raise RuntimeError("group_norm_nhwc expects channels-last input (stride 1 along dim 1)")
     nd = x.dim()
@@ -482,6 +538,11 @@ def group_norm_nhwc(x, weight, bias, num_groups, eps=1e-5, activation="identity"
     def unflat(t):
         return t.permute(0, 2, 1).reshape(shape).permute(0, nd - 1, *range(1, nd - 1))
 
+    if out_dtype is not None and out_dtype != x.dtype:
+        if residual is not None or channel_bias is not None or return_sum:
+            raise RuntimeError("out_dtype cannot be combined with residual / channel_bias / return_sum")
+        Y, _means, _rstds = torch.ops.gnop.fwd_cast(X_flat, weight, bias, num_groups, eps, code, out_dtype)
+        return unflat(Y)
     if residual is None and channel_bias is None and not return_sum:
         Y, _means, _rstds = torch.ops.gnop.fwd(X_flat, weight, bias, num_groups, eps, code)
         return unflat(Y)
@@ -564,12 +625,24 @@ _TORCH_ACTIVATIONS = (
 class GN_NHWC(nn.GroupNorm):
     """custom_gn.py:49-90.  GroupNorm over channels-last input with the activation applied in the same pass."""
 
-    def __init__(self, num_groups, num_channels, activation="identity", **kwargs):
+    def __init__(self, num_groups, num_channels, activation="identity", out_dtype=None, **kwargs):
         super().__init__(num_groups, num_channels, **kwargs)
         self.activation = activation
         self.act_code = ACTIVATION_CODES[activation]  # unknown name -> KeyError, as in the reference
+        # not in the reference: the type the result leaves in (None: the input's).  float32 channels-last device input
+        # is written as float16 / bfloat16 by the kernel itself; any other combination is converted afterwards.
+        self.out_dtype = out_dtype
 
     def forward(self, x):
+        if self.out_dtype is not None and self.out_dtype != x.dtype:
+            if (x.is_cuda and x.dtype == torch.float32 and x.stride(1) == 1
+                    and self.out_dtype in (torch.float16, torch.bfloat16)):
+                return group_norm_nhwc(x, self.weight, self.bias, self.num_groups, self.eps, self.activation,
+                                       out_dtype=self.out_dtype)
+            return self._forward_same_dtype(x).to(self.out_dtype)
+        return self._forward_same_dtype(x)
+
+    def _forward_same_dtype(self, x):
         # The reference wraps this method in torch._dynamo.disable (custom_gn.py:63): its operators cannot be traced,
         # so a compiled model breaks its graph here.  These operators can (meta kernels + registered autograd), so
         # under torch.compile the same computation is expressed through them and stays inside the caller's graph.

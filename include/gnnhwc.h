@@ -103,6 +103,26 @@ int gnnhwc_fwd(const void *x, const void *weight, const void *bias,
                void *workspace, size_t workspace_bytes, void *stream /* hipStream_t */);
 
 /*
+ * Forward of float data with y written in a 16-bit type (no counterpart in the reference, where y has the type of x,
+ * custom_gn.cpp:28, and the cast for a half-precision consumer is a separate elementwise pass).  For the
+ * GroupNorm -> activation -> convolution step of a network whose convolutions run in half precision on a float
+ * residual stream: y leaves in the convolution's type, each value rounded once from the fp32 result, so the forward
+ * writes S/2 instead of S bytes and the cast kernel (1.5 S more traffic) disappears.
+ *   dtype   : GNNHWC_F32 (type of x).
+ *   y_dtype : GNNHWC_F16 or GNNHWC_BF16 (type of y); GNNHWC_F32 makes this gnnhwc_fwd.  Anything else, or another
+ *             dtype with a y_dtype different from it, is GNNHWC_ERR_INVALID_ARGUMENT.
+ * y must not be the buffer of x when the types differ.  Everything else as gnnhwc_fwd (same workspace size).
+ * A backward that follows takes dy in dtype: gnnhwc_bwd has one element type, so a 16-bit incoming gradient is
+ * widened by the caller first.
+ */
+int gnnhwc_fwd_cast(const void *x, const void *weight, const void *bias,
+                    void *y, void *mean, void *rstd,
+                    int64_t N, int64_t R, int64_t C, int64_t G,
+                    double eps, int act,
+                    int dtype, int param_dtype, int stats_dtype, int y_dtype,
+                    void *workspace, size_t workspace_bytes, void *stream /* hipStream_t */);
+
+/*
  * Forward with the additions that precede the normalisation fused in (no counterpart in the reference, whose
  * callers add in a separate pass: in a diffusion ResNet block `h + temb[:, :, None, None]` before the second
  * norm, and `shortcut + h` before the next block's first norm).  The tensor that is normalised is
