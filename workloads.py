@@ -40,9 +40,13 @@ for _dt in ("fp32", "bf16"):
 SD_UNET_SWEEP = ("c3a", "c3b", "c3c")
 ALL_NAMES = tuple(CONFIGS)
 
+# Measured by bench.py --nchw only (not a parity configuration of its own; tests/test_gpu_nchw.py has its small relatives):
+# one group of many long rows, the channels-first case where a slab has thousands of partial sums.
+EXTRA = {"one_group": Config("one_group", "bf16", (1, 512, 256, 256), 1, "silu", "fwd+bwd", "normal")}
+
 
 def _seed(name):
-    return 1000 + ALL_NAMES.index(name)
+    return 1000 + ALL_NAMES.index(name) if name in ALL_NAMES else 2000 + sorted(EXTRA).index(name)
 
 
 def make_inputs(cfg, device="cpu", shape=None):
