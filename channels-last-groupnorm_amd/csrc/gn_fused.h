@@ -224,8 +224,8 @@ __device__ __forceinline__ void for_group_records(const SyncArea &s, __amdgpu_bu
 // ---------------------------------------------------------------------------------------------
 // Resident forward.  NV = register capacity in rows per lane.  Statistics follow the same definitions
 // as the streaming kernels (count / mean / M2, biased variance, rstd = 1 / sqrt(var + eps);
-// src/gnnhwc/csrc/Welford.h:8-21,66-72, gn_kernel.cu:175,254,291); with the whole tile in registers
-// the per-lane moments are an exact two-pass computation.
+// src/gnnhwc/csrc/Welford.h:8-21,66-72, gn_kernel.cu:175,254,291); the per-lane moments are taken in one pass, as
+// sums about the lane's own first row.
 //   records : {mean, M2, epoch} per (n, chunk, group, tile)
 // ---------------------------------------------------------------------------------------------
 // ADD: 0 plain forward; 1 a per-(sample, channel) addend only (same register budget as the plain kernel);
