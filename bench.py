@@ -61,7 +61,8 @@ def parse_args():
     ap.add_argument("--timeline", action="store_true",
                     help="no headline: print the in-kernel timeline of the single-launch kernels (wall-clock stamps every workgroup "
                          "takes at its phase boundaries; min / median / max over the workgroups of one launch) for each shape of "
-                         "the workload (default here: c3a c3b c3c c4a), forward and backward")
+                         "the workload (default here: c3a c3b c3c c4a), forward and backward, in a loop over that shape alone; "
+                         "for the default workload first the same inside the sweep itself")
     ap.add_argument("--counter-workload", action="store_true",
                     help="no timing: one 256 MiB plain copy (calibration) and a few fwd+bwd calls per shape, for a rocprofv3 --pmc run")
     return ap.parse_args()
@@ -368,6 +369,61 @@ def timeline(names, device, reps=5):
         torch.cuda.empty_cache()
 
 
+def timeline_in_sweep(names, device, reps=5):
+    """The same stamps for every single-launch kernel of a workload taken INSIDE the workload: a few full steps run, then
+    the launches of one more step up to and including the traced one, so that the traced launch finds the caches and
+    the queue as it does in the timed region (its tensors evicted by the other shapes, another kernel ahead of it)."""
+    import numpy as np
+    import torch
+    from gnnhwc import _cabi
+    import workloads as configs
+
+    stream = torch.cuda.current_stream().cuda_stream
+    words = np.zeros((1024, 8), dtype=np.uint64)
+    probs = [Problem(configs.CONFIGS[n], device) for n in names]
+    launches = [(p, w) for p in probs for w in (("fwd", "bwd") if p.bwd else ("fwd",))]
+    ev = {n: {k: us for k, (us, _) in kinds.items()} for n, kinds in kernel_profile(probs, 50).items()}
+    print("# in-kernel timeline inside the workload %s, microseconds after the first workgroup of the launch started: "
+          "min / median / max over workgroups" % "+".join(names))
+    for ti, (p, which) in enumerate(launches):
+        stamps = FWD_STAMPS if which == "fwd" else BWD_STAMPS
+        kind = "fused_fwd" if which == "fwd" else "fused_bwd"
+        evs = ev.get(p.cfg.name, {})
+        if kind not in evs:
+            print("%s %s: multi-launch kernels (no in-kernel timeline); event-timed in the workload: %s"
+                  % (p.cfg.name, which, ", ".join("%s %.2f us" % kv for kv in evs.items() if not kv[0].startswith("fused"))))
+            continue
+        rows = []
+        for _ in range(reps):
+            torch.cuda.synchronize()
+            time.sleep(0.002)
+            for _ in range(6):
+                for q, w in launches:
+                    q.step(0, stream, w)
+            for q, w in launches[:ti + 1]:
+                q.step(0, stream, w)
+            torch.cuda.synchronize()
+            _cabi.check(_cabi.lib.gnnhwc_debug_read_trace(words.ctypes.data, words.size), "gnnhwc_debug_read_trace")
+            t = words.astype(np.int64)
+            live = t[:, 0] >= t[:, 0].max() - 300
+            t = t[live]
+            rel = (t - t[:, 0].min()) / 100.0
+            taken = {}
+            for pt, _ in stamps:
+                v = rel[:, pt][t[:, pt] >= t[:, 0].min()]
+                if v.size:
+                    taken[pt] = (float(v.min()), float(np.median(v)), float(v.max()))
+            rows.append((int(live.sum()), taken))
+        print("%s %s: %d workgroups in the traced launch; event-timed in the workload: %s %.2f us"
+              % (p.cfg.name, which, rows[-1][0], kind, evs[kind]))
+        for pt, label in stamps:
+            vals = [r[1][pt] for r in rows if pt in r[1]]
+            if not vals:
+                continue
+            med = [statistics.median(v[i] for v in vals) for i in range(3)]
+            print("    %-58s %7.2f / %7.2f / %7.2f" % (label, med[0], med[1], med[2]))
+
+
 def cpu_baseline(cfg_names, seconds):
     """torch's CPU GroupNorm + activation + autograd on the host cores, same seeded tensors and dtype."""
     import torch
@@ -621,6 +677,8 @@ def main():
     torch.cuda.set_device(device)
     use_graph = args.graph
     if args.timeline:
+        if args.workload == "sd_unet":
+            timeline_in_sweep(list(configs.SD_UNET_SWEEP), device)
         timeline(["c3a", "c3b", "c3c", "c4a"] if args.workload == "sd_unet" else
                  list(configs.ALL_NAMES) if args.workload == "all" else [args.workload], device)
         return

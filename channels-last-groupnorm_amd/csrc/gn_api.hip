@@ -345,6 +345,9 @@ bool trace_waits() {
   return w;
 }
 unsigned long long *trace_buffer() {
+#if !GN_TRACE
+  return nullptr;  // this build's kernels have no stamps
+#endif
   static unsigned long long *buf = []() -> unsigned long long * {
     if (env_int("GNNHWC_TRACE", 0) == 0) return nullptr;
     void *p = nullptr;
@@ -671,6 +674,10 @@ int gnnhwc_debug_set_spin_limit(int polls) {
 }
 
 int gnnhwc_debug_read_trace(unsigned long long *out, int64_t count) {
+#if !GN_TRACE
+  return fail(GNNHWC_ERR_INVALID_ARGUMENT, "this library is built without trace points: load libgnnhwc_hip_trace.so "
+              "(the Python binding does when GNNHWC_TRACE is set in the environment)");
+#endif
   unsigned long long *buf = trace_buffer();
   if (!buf) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "tracing is off (set GNNHWC_TRACE=1 before the first call)");
   const int64_t cap = (int64_t)kMaxResidentBlocks * 8;

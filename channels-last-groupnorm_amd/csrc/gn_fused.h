@@ -55,6 +55,7 @@ struct SyncArea {
 };
 constexpr int kTracePoints = 8;
 __device__ __forceinline__ void trace_point(const SyncArea &s, int point, float after = 0.f) {
+#if GN_TRACE
   if (!s.trace) return;
   // either stamp a phase once its memory operations have completed, or (trace_wait == 0) leave the kernel's
   // own overlap alone and only order the stamp behind the value `after`
@@ -64,6 +65,11 @@ __device__ __forceinline__ void trace_point(const SyncArea &s, int point, float 
     const int64_t b = ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
     if (b < kMaxResidentBlocksDev) s.trace[b * kTracePoints + point] = wall_clock64();
   }
+#else
+  (void)s;
+  (void)point;
+  (void)after;
+#endif
 }
 
 // A launch recorded into a HIP graph is replayed with identical kernel arguments, so the host cannot give
@@ -330,30 +336,22 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
     LV::unpack(buf[0], k);
 #pragma unroll
     for (int j = 0; j < VEC; ++j) { s1[j] = (A)0; s2[j] = (A)0; }
-    if (rows == NV) {  // a full tile (all but the last tile of a sample): no masking of rows past the lane's last one
+    // rows past the lane's last one (only in the last tile of a sample) are replaced by the pivot row, whose deviation
+    // is exactly zero: one loop serves full and partial tiles, and a full tile only skips this block
+    if (rows != NV) {
 #pragma unroll
-      for (int u = 1; u < NV; ++u) {
-        A v[VEC];
-        LV::unpack(buf[u], v);
+      for (int u = 1; u < NV; ++u)
+        if (u >= rows) buf[u] = buf[0];
+    }
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) {
-          const A d = v[j] - k[j];
-          s1[j] += d;
-          s2[j] += d * d;
-        }
-      }
-    } else {
+    for (int u = 1; u < NV; ++u) {
+      A v[VEC];
+      LV::unpack(buf[u], v);
 #pragma unroll
-      for (int u = 1; u < NV; ++u) {
-        const bool keep = u < rows;
-        A v[VEC];
-        LV::unpack(buf[u], v);
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) {
-          const A d = keep ? v[j] - k[j] : (A)0;
-          s1[j] += d;
-          s2[j] += d * d;
-        }
+      for (int j = 0; j < VEC; ++j) {
+        const A d = v[j] - k[j];
+        s1[j] += d;
+        s2[j] += d * d;
       }
     }
     const A inv = fast_rcp((A)rows);
@@ -543,42 +541,29 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
       lane_coeffs<A, VEC, false>(p, l, sm_mu, sm_rs, nullptr, nullptr, sa, sb, c1, c2);
       // dy is not needed again: its registers keep g' = dy * act'(z) for the dx phase (for 16-bit data
       // rounded to T, the rounding an unfused activation backward applies to the same quantity).
-      // A full tile (all but the last tile of a sample) needs no masking of rows past the lane's last one.
-      if (rows == NV) {
+      // Rows past the lane's last one (only in the last tile of a sample; they re-read a valid row of x) get dy = 0,
+      // hence g' = 0 and no contribution: one loop serves full and partial tiles, and a full tile only skips this block.
+      if (rows != NV) {
+        const typename LV::raw_t zero = {};
 #pragma unroll
-        for (int u = 0; u < NV; ++u) {
-          A vx[VEC], vd[VEC];
-          pin(bx[u]);  // one row at a time: cheap activations otherwise tempt the scheduler into unpacking many
-          pin(bd[u]);  // rows ahead, which costs more registers than the tile itself
-          LV::unpack(bx[u], vx);
-          LV::unpack(bd[u], vd);
+        for (int u = 0; u < NV; ++u)
+          if (u >= rows) bd[u] = zero;
+      }
 #pragma unroll
-          for (int j = 0; j < VEC; ++j) {
-            const A g = vd[j] * act_bwd<ACT, A>(vx[j] * sa[j] + sb[j]);
-            s1[j] += g * vx[j];
-            s2[j] += g;
-            vd[j] = g;
-          }
-          bd[u] = LV::pack(vd);
+      for (int u = 0; u < NV; ++u) {
+        A vx[VEC], vd[VEC];
+        pin(bx[u]);  // one row at a time: cheap activations otherwise tempt the scheduler into unpacking many
+        pin(bd[u]);  // rows ahead, which costs more registers than the tile itself
+        LV::unpack(bx[u], vx);
+        LV::unpack(bd[u], vd);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const A g = vd[j] * act_bwd<ACT, A>(vx[j] * sa[j] + sb[j]);
+          s1[j] += g * vx[j];
+          s2[j] += g;
+          vd[j] = g;
         }
-      } else {
-#pragma unroll
-        for (int u = 0; u < NV; ++u) {
-          const A keep = u < rows ? (A)1 : (A)0;
-          A vx[VEC], vd[VEC];
-          pin(bx[u]);
-          pin(bd[u]);
-          LV::unpack(bx[u], vx);
-          LV::unpack(bd[u], vd);
-#pragma unroll
-          for (int j = 0; j < VEC; ++j) {
-            const A g = keep * vd[j] * act_bwd<ACT, A>(vx[j] * sa[j] + sb[j]);
-            s1[j] += g * vx[j];
-            s2[j] += g;
-            vd[j] = g;
-          }
-          bd[u] = LV::pack(vd);
-        }
+        bd[u] = LV::pack(vd);
       }
     }
     trace_point(sync, 6, (float)(s1[0] + s2[0]));

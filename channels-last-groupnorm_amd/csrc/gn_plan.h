@@ -3,6 +3,12 @@
 // (src/gnnhwc/csrc/gn_kernel.cu:37-60,121-128) but is built around 128-bit lane vectors and
 // 256-thread workgroups instead of <=128-thread blocks over a virtual H x W factorisation.
 #pragma once
+// GN_TRACE = 1 compiles the phase stamps of the single-launch kernels in (libgnnhwc_hip_trace.so).  The library proper is
+// built without them: even switched off at run time they cost registers, basic-block boundaries and code on the path
+// every launch executes (measured: 2 % of the SD-UNet sweep).
+#ifndef GN_TRACE
+#define GN_TRACE 0
+#endif
 #include <stdint.h>
 
 namespace gn {

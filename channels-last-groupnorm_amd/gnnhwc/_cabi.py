@@ -8,7 +8,10 @@ import ctypes
 import os
 
 _CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
-LIB_PATH = os.path.join(_CSRC, "libgnnhwc_hip.so")
+# With GNNHWC_TRACE set (1 or 2) at import, the twin library with the in-kernel phase stamps compiled in is loaded instead
+# (bench.py --timeline); the library proper carries no trace code at all.
+TRACING = os.environ.get("GNNHWC_TRACE", "0") not in ("", "0")
+LIB_PATH = os.path.join(_CSRC, "libgnnhwc_hip_trace.so" if TRACING else "libgnnhwc_hip.so")
 
 # dtype / activation codes of include/gnnhwc.h
 F32, F64, F16, BF16 = 0, 1, 2, 3

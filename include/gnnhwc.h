@@ -278,10 +278,12 @@ int gnnhwc_debug_plan(int64_t N, int64_t R, int64_t C, int64_t G, int dtype, int
 
 /*
  * In-kernel timeline of the single-launch kernels, for tuning (no counterpart in the reference; its
- * nearest relative is the DEBUG(...) launch-parameter printf, gn_kernel.cu:13-19).  With GNNHWC_TRACE=1
- * in the environment at the first call, thread 0 of every workgroup of a single-launch kernel writes a
- * 100 MHz wall-clock stamp at up to 8 phase boundaries.  This call synchronises the device and copies
- * `count` 64-bit words, laid out [workgroup][8], from the most recent such launch.
+ * nearest relative is the DEBUG(...) launch-parameter printf, gn_kernel.cu:13-19).  Only in
+ * libgnnhwc_hip_trace.so, the same library compiled with the stamps (the library proper has none: even switched
+ * off they cost every launch time, and there this call returns an error).  With GNNHWC_TRACE=1 (stamps wait for
+ * outstanding memory operations) or 2 (they do not) in the environment at the first call, thread 0 of every
+ * workgroup of a single-launch kernel writes a 100 MHz wall-clock stamp at up to 8 phase boundaries.  This call
+ * synchronises the device and copies `count` 64-bit words, laid out [workgroup][8], from the most recent such launch.
  */
 int gnnhwc_debug_read_trace(unsigned long long *out, int64_t count);
 

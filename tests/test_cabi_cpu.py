@@ -29,6 +29,12 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(_cabi.LIB_PATH)
     for n in names:
         assert hasattr(lib, n), n
+    # the twin built with the in-kernel phase stamps (loaded instead when GNNHWC_TRACE is set) exports the same interface
+    twin = ctypes.CDLL(os.path.join(os.path.dirname(_cabi.LIB_PATH), "libgnnhwc_hip_trace.so"))
+    for n in names:
+        assert hasattr(twin, n), n
+    if not _cabi.TRACING:  # the library proper has no stamps to read
+        assert _cabi.lib.gnnhwc_debug_read_trace(None, 8) == -1 and "trace" in _cabi.last_error()
 
 
 def test_version_and_kind_names():
