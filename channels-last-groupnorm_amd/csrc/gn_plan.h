@@ -23,24 +23,36 @@ constexpr int kNumCU = 256;         // MI355X
 constexpr int kTargetBlocks = 768;  // ~3 workgroups per CU, what the streaming kernels' registers allow: one resident wave
 constexpr int kEarly = 4;            // tile partials a lane of a consumer workgroup fetches ahead of its data
 
-// Division by a launch constant without the integer-division sequence (a few dozen instructions on this
-// hardware, all of them latency in a workgroup's prologue): q = umulhi(n, magic) with
-// magic = floor(2^32 / d) + 1 is exact for 0 <= n with n d < 2^32.  The host fills `magic` only when the
-// largest dividend it will see satisfies that; magic == 0 selects the ordinary division.
+// Division by a launch constant without the integer-division sequence (a few dozen instructions on this hardware, all
+// of them latency in a workgroup's prologue) and without a branch: with L = ceil(log2 d) and
+// magic = floor(2^32 (2^L - d) / d) + 1,
+//   t = umulhi(magic, n),   n / d = (t + ((n - t) >> min(L, 1))) >> max(L - 1, 0)
+// for every 0 <= n < 2^32 and 1 <= d < 2^31 (Granlund and Montgomery, "Division by invariant integers using
+// multiplication", 1994, section 4).  No fallback means no cold code and no extra basic blocks in the kernels.
 struct Divisor {
   int d;
   unsigned magic;
+  int sh1, sh2;
 };
-inline Divisor make_divisor(int64_t d, int64_t max_n) {
+__host__ __device__ inline Divisor make_divisor(int64_t d, int64_t /*largest dividend: any value below 2^32 is fine*/) {
   Divisor v;
   v.d = (int)d;
-  v.magic = 0;
-  if (d > 1 && max_n >= 0 && max_n < ((int64_t)1 << 32) / d) v.magic = (unsigned)((((uint64_t)1) << 32) / (uint64_t)d + 1);
+  const uint64_t ud = (uint64_t)(d < 1 ? 1 : d);
+  int L = 0;
+  while (((uint64_t)1 << L) < ud) ++L;
+  v.magic = (unsigned)(((((uint64_t)1 << L) - ud) << 32) / ud + 1);
+  v.sh1 = L < 1 ? L : 1;
+  v.sh2 = L > 1 ? L - 1 : 0;
   return v;
 }
-__device__ __forceinline__ int div_by(int n, const Divisor &v) {
-  if (v.magic) return (int)__umulhi((unsigned)n, v.magic);
-  return v.d == 1 ? n : n / v.d;
+__host__ __device__ __forceinline__ int div_by(int n, const Divisor &v) {
+  const unsigned un = (unsigned)n;
+#if defined(__HIP_DEVICE_COMPILE__)
+  const unsigned t = __umulhi(v.magic, un);
+#else
+  const unsigned t = (unsigned)(((uint64_t)v.magic * un) >> 32);
+#endif
+  return (int)((t + ((un - t) >> v.sh1)) >> v.sh2);
 }
 
 // One workgroup owns `tile_rows` consecutive rows of one sample and one chunk of `lpr` lane vectors
