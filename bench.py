@@ -63,6 +63,9 @@ def parse_args():
                          "takes at its phase boundaries; min / median / max over the workgroups of one launch) for each shape of "
                          "the workload (default here: c3a c3b c3c c4a), forward and backward, in a loop over that shape alone; "
                          "for the default workload first the same inside the sweep itself")
+    ap.add_argument("--switch-cost", action="store_true",
+                    help="no headline: event-timed duration of each kernel of the workload when it follows itself and when it "
+                         "follows a different kernel whose data is tiny (a 1 MB plain copy; a small GroupNorm forward)")
     ap.add_argument("--counter-workload", action="store_true",
                     help="no timing: one 256 MiB plain copy (calibration) and a few fwd+bwd calls per shape, for a rocprofv3 --pmc run")
     return ap.parse_args()
@@ -424,6 +427,59 @@ def timeline_in_sweep(names, device, reps=5):
             print("    %-58s %7.2f / %7.2f / %7.2f" % (label, med[0], med[1], med[2]))
 
 
+def switch_cost(names, device):
+    """What following a DIFFERENT kernel costs a launch.  Each kernel of the workload is timed (event pair bound to the
+    dispatch) in three loops: relaunched back to back; alternating with the library's plain copy kernel on 1 MB; and
+    alternating with a GroupNorm forward on a 1 MB tensor.  The other kernels touch too little data to evict the timed
+    kernel's tensors from the caches, so the difference is what the switch itself costs (a new program on every CU)."""
+    import torch
+    from gnnhwc import _cabi
+    import workloads as configs
+
+    stream = torch.cuda.current_stream().cuda_stream
+    src = torch.empty((1 << 20,), dtype=torch.uint8, device=device)
+    dst = torch.empty_like(src)
+    small = Problem(configs.CONFIGS["c5a_bf16_gelu"], device)
+
+    def copy():
+        _cabi.check(_cabi.lib.gnnhwc_debug_copy(dst.data_ptr(), src.data_ptr(), src.numel(), stream), "gnnhwc_debug_copy")
+
+    others = (("after itself", None), ("after a 1 MB plain copy", copy),
+              ("after a 1 MB GroupNorm forward", lambda: small.step(0, stream, "fwd")))
+    print("# event-timed microseconds per launch; same buffers every launch")
+    print("%-6s %-4s %-12s %14s %26s %32s" % ("shape", "pass", "kernel", others[0][0], others[1][0], others[2][0]))
+    for name in names:
+        p = Problem(configs.CONFIGS[name], device)
+        for which in (("fwd", "bwd") if p.bwd else ("fwd",)):
+            row, kind = [], None
+            for _, other in others:
+                def it(profile):
+                    if other is not None:
+                        other()
+                    _cabi.profile_enable(profile)
+                    p.step(0, stream, which)
+                    _cabi.profile_enable(False)
+                for _ in range(50):
+                    it(False)
+                torch.cuda.synchronize()
+                for _ in range(20):
+                    it(True)
+                _cabi.profile_collect()
+                best = None
+                for _ in range(3):
+                    for _ in range(100):
+                        it(True)
+                    torch.cuda.synchronize()
+                    res = {k: ms / n * 1e3 for k, (n, ms) in _cabi.profile_collect().items() if n}
+                    kind = "+".join(sorted(res))
+                    v = sum(res.values())
+                    best = v if best is None else min(best, v)
+                row.append(best)
+            print("%-6s %-4s %-12s %14.2f %26.2f %32.2f" % (name, which, kind, row[0], row[1], row[2]))
+        del p
+        torch.cuda.empty_cache()
+
+
 def cpu_baseline(cfg_names, seconds):
     """torch's CPU GroupNorm + activation + autograd on the host cores, same seeded tensors and dtype."""
     import torch
@@ -676,6 +732,10 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
     use_graph = args.graph
+    if args.switch_cost:
+        switch_cost(list(configs.SD_UNET_SWEEP) if args.workload == "sd_unet" else
+                    list(configs.ALL_NAMES) if args.workload == "all" else [args.workload], device)
+        return
     if args.timeline:
         if args.workload == "sd_unet":
             timeline_in_sweep(list(configs.SD_UNET_SWEEP), device)
