@@ -369,6 +369,28 @@ template <typename A> __device__ __forceinline__ void segment_sum2(A &a, A &b, i
     b += ob;
   }
 }
+// The same for callers that need the totals in ONE lane of the segment only: segment_leader(width).  Up to a row of 16
+// lanes this is the butterfly above; the steps across rows are DPP row broadcasts (lane 15 of a row into the next
+// row, lane 31 into the upper half of the wavefront), which cost one addition each where the butterfly's cross-row
+// exchanges go through the LDS crossbar (an address computation, a permute and a wait per value and step).
+constexpr int kDppRowBcast15 = 0x142, kDppRowBcast31 = 0x143;
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ float dpp_rows_add(float v) {
+  const int i = __builtin_bit_cast(int, v);
+  return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, i, CTRL, ROW_MASK, 0xF, false));
+}
+__device__ __forceinline__ void segment_reduce2(float &a, float &b, int width) {
+  if (width >= 2) { a += dpp_move<kDppQuadXor1>(a); b += dpp_move<kDppQuadXor1>(b); }
+  if (width >= 4) { a += dpp_move<kDppQuadXor2>(a); b += dpp_move<kDppQuadXor2>(b); }
+  if (width >= 8) { a += dpp_move<kDppRowHalfMirror>(a); b += dpp_move<kDppRowHalfMirror>(b); }
+  if (width >= 16) { a += dpp_move<kDppRowMirror>(a); b += dpp_move<kDppRowMirror>(b); }
+  if (width >= 32) { a = dpp_rows_add<kDppRowBcast15, 0xA>(a); b = dpp_rows_add<kDppRowBcast15, 0xA>(b); }
+  if (width >= 64) { a = dpp_rows_add<kDppRowBcast31, 0xC>(a); b = dpp_rows_add<kDppRowBcast31, 0xC>(b); }
+}
+__device__ __forceinline__ void segment_reduce2(double &a, double &b, int width) { segment_sum2(a, b, width); }
+// Lane (inside its segment) that holds the totals after segment_reduce2.
+template <typename A> __device__ __forceinline__ int segment_leader(int width) {
+  return sizeof(A) == 4 && width >= 32 ? width - 1 : 0;
+}
 // Segment index of a thread when the workgroup is cut into segments of L lanes (a power of two <= 64), numbered so that
 // consecutive segments sit in DIFFERENT wavefronts: the first few groups of a chunk then keep all four SIMDs of the CU
 // busy instead of queueing in the first wavefront.

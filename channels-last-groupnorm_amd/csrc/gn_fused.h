@@ -139,14 +139,14 @@ __device__ __forceinline__ float poison() { return __builtin_nanf(""); }
 // the group starts -- with all 256 lanes, and published as one final record per (sample, group) that everybody polls.
 // One more round trip, a few thousand times less traffic.
 __device__ __forceinline__ bool owns_group(const Plan &p, const LanePos &l, int gi) {
-  return (l.g_lo + gi) * p.D >= l.cstart && gi % p.tiles == l.tile;
+  return (l.g_lo + gi) * p.D >= l.cstart && gi - div_by(gi, p.by_tiles) * p.tiles == l.tile;
 }
 // Sum of two values over the 256 lanes of the workgroup (fixed tree: wavefront, then the four wavefronts in order);
 // every lane gets the result.  Uses 8 floats of LDS at `scratch`; the caller's other LDS data is not touched.
 template <typename A> __device__ __forceinline__ void block_sum2(A &a, A &b, A *scratch) {
-  segment_sum2(a, b, 64);
+  segment_reduce2(a, b, 64);
   __syncthreads();  // scratch may still be read from a previous use
-  if ((threadIdx.x & 63) == 0) {
+  if ((int)(threadIdx.x & 63) == segment_leader<A>(64)) {
     scratch[threadIdx.x >> 6] = a;
     scratch[4 + (threadIdx.x >> 6)] = b;
   }
@@ -442,8 +442,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
       const A K = __shfl(mean_l, (int)(threadIdx.x & 63 & ~(L - 1)), 64);
       const A d = mean_l - K;
       A t1 = nl * d, t2 = m2_l + nl * d * d;
-      segment_sum2(t1, t2, L);
-      if (valid && sl == 0) {
+      segment_reduce2(t1, t2, L);
+      if (valid && sl == segment_leader<A>(L)) {
         const A dm = t1 * fast_rcp(total);
         const A gmean = K + dm;
         const A rs = fast_rsqrt((t2 - t1 * dm) * fast_rcp(total) + eps);
@@ -601,8 +601,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
       if (valid) group_span(p, l, g, ca, cb);
       A ta = (A)0, tb = (A)0;
       for (int c = ca + sl; c < cb; c += L) { ta += sm1[c]; tb += sm2[c]; }
-      segment_sum2(ta, tb, L);
-      if (valid && sl == 0) record_store(rb, record_slot(q, p.G, (int)n, l.tile, l.chunk, g), ta, tb, sync.epoch);
+      segment_reduce2(ta, tb, L);
+      if (valid && sl == segment_leader<A>(L)) record_store(rb, record_slot(q, p.G, (int)n, l.tile, l.chunk, g), ta, tb, sync.epoch);
     }
   }
   __syncthreads();
@@ -647,8 +647,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
         ta += ra;
         tb += rbv;
       });
-      segment_sum2(ta, tb, L);
-      if (valid && sl == 0) {
+      segment_reduce2(ta, tb, L);
+      if (valid && sl == segment_leader<A>(L)) {
         const A mu = sm_mu[gi];
         const A rs = sm_rs[gi];
         const A s = fast_rcp((A)p.D * (A)p.R);
@@ -681,7 +681,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
 #pragma unroll
     for (int i = 0; i < kTailFast; ++i) {
       const int e = tsl + i * TL;
-      const int nn = e < pairs ? e / p.tiles : 0;
+      const int nn = e < pairs ? div_by(e, p.by_tiles) : 0;
       const int t = e < pairs ? e - nn * p.tiles : 0;
       trec[i] = record_load(rbc, __mul24(__mul24(nn, p.tiles) + t, (int)p.C) + tail_c);
       tmu[i] = load_scalar_flat<A>(mean_all, nn * p.G + tail_g, sdtype, safe);
@@ -729,7 +729,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
       A t1 = (A)0, t2 = (A)0;
       // one (sample, tile) pair: wait until its record is this launch's (if it is this launch's to write) and add it
       auto add = [&](int e, u32x4 rec, A mu, A rs) {
-        const int64_t nn = e / p.tiles;
+        const int64_t nn = div_by(e, p.by_tiles);
         const int t = e - (int)nn * p.tiles;
         while (valid && nn >= n0 && (!record_ready(rec, sync.epoch) || sync.max_spins == kForcedTimeout)) {
           if (++spins > sync.max_spins) {
@@ -755,14 +755,14 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
         }
       }
       for (; e < pairs; e += TL) {
-        const int64_t nn = e / p.tiles;
+        const int64_t nn = div_by(e, p.by_tiles);
         const int t = e - (int)nn * p.tiles;
         add(e, record_load(rbc, (nn * p.tiles + t) * p.C + c), load_scalar<A>(mean_all, nn * p.G + g, sdtype),
             load_scalar<A>(rstd_all, nn * p.G + g, sdtype));
       }
       if (!valid) { t1 = (A)0; t2 = (A)0; }
-      segment_sum2(t1, t2, TL);
-      if (valid && tsl == 0) {
+      segment_reduce2(t1, t2, TL);
+      if (valid && tsl == segment_leader<A>(TL)) {
         if (dw) store_param<PT, A>(dw, c, t1);
         if (db) store_param<PT, A>(db, c, t2);
       }

@@ -1009,7 +1009,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
       const int c = cstart + cbase + cl;
       A t1 = (A)0, t2 = (A)0;
       if (cbase + cl < wch && ts < nsl) {
-        const int g = c / p.D;
+        const int g = div_by(c, p.by_D);
         for (int64_t n = 0; n < p.N; ++n) {
           A s1 = (A)0, s2 = (A)0;
           for (int t = ts; t < q.tiles; t += nsl) {
