@@ -690,20 +690,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
   }
   trace_point(sync, 3);
   if (rows > 0) {
-    {
-      int gi = div_by(l.cvi * VEC, p.by_D);
-      int rem = l.cvi * VEC - gi * p.D;
-      gi -= l.g_lo;
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        c1[j] = sm1[gi];
-        c2[j] = sm2[gi];
-        ++rem;
-        const bool wrap = rem == p.D;
-        rem = wrap ? 0 : rem;
-        gi += wrap ? 1 : 0;
-      }
-    }
+    lane_group_pairs<A, VEC>(p, l, sm1, sm2, c1, c2);
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
       if (u < rows) {

@@ -668,27 +668,50 @@ template <int VEC> __device__ __forceinline__ SafeLane safe_lane(const Plan &p, 
 // a = rstd * gamma, b = beta - mean * a: normalise + affine as one FMA per element (same folding as
 // src/gnnhwc/csrc/gn_kernel.cu:350-379, 601-602, 783-784).  Group statistics come from LDS; optional
 // per-group extras (the backward's coef1 / coef2) are fetched alongside.  On return sa / sb replace gamma / beta.
-template <typename A, int VEC, bool EXTRA>
-__device__ __forceinline__ void lane_coeffs(const Plan &p, const LanePos &l, const A *sm_mu, const A *sm_rs,
-                                            const A *sm_c1, const A *sm_c2, A (&sa)[VEC], A (&sb)[VEC], A (&c1)[VEC],
-                                            A (&c2)[VEC]) {
+// Per-channel copies of two per-group LDS arrays (indexed by group inside the chunk) for the lane's VEC channels.
+// When a group has at least VEC channels the lane's channels lie in at most two groups: four LDS reads and a select
+// per channel instead of two reads and the bookkeeping of the group boundary per channel.
+template <typename A, int VEC>
+__device__ __forceinline__ void lane_group_pairs(const Plan &p, const LanePos &l, const A *sm_a, const A *sm_b, A (&va)[VEC],
+                                                 A (&vb)[VEC]) {
   const int c = l.cvi * VEC;
   int gi = div_by(c, p.by_D);
   int rem = c - gi * p.D;
   gi -= l.g_lo;
+  if (VEC > 1 && p.D >= VEC) {
+    const int split = p.D - rem;               // channels j < split lie in group gi, the others in gi + 1
+    const int gj = split < VEC ? gi + 1 : gi;  // (no second group: read the first again, never past the chunk's groups)
+    const A a0 = sm_a[gi], b0 = sm_b[gi], a1 = sm_a[gj], b1 = sm_b[gj];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const bool first = j < split;
+      va[j] = first ? a0 : a1;
+      vb[j] = first ? b0 : b1;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      va[j] = sm_a[gi];
+      vb[j] = sm_b[gi];
+      ++rem;
+      const bool wrap = rem == p.D;
+      rem = wrap ? 0 : rem;
+      gi += wrap ? 1 : 0;
+    }
+  }
+}
+template <typename A, int VEC, bool EXTRA>
+__device__ __forceinline__ void lane_coeffs(const Plan &p, const LanePos &l, const A *sm_mu, const A *sm_rs,
+                                            const A *sm_c1, const A *sm_c2, A (&sa)[VEC], A (&sb)[VEC], A (&c1)[VEC],
+                                            A (&c2)[VEC]) {
+  A mu[VEC], rs[VEC];
+  lane_group_pairs<A, VEC>(p, l, sm_mu, sm_rs, mu, rs);
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
-    sa[j] = sm_rs[gi] * sa[j];
-    sb[j] = sb[j] - sm_mu[gi] * sa[j];
-    if (EXTRA) {
-      c1[j] = sm_c1[gi];
-      c2[j] = sm_c2[gi];
-    }
-    ++rem;
-    const bool wrap = rem == p.D;
-    rem = wrap ? 0 : rem;
-    gi += wrap ? 1 : 0;
+    sa[j] = rs[j] * sa[j];
+    sb[j] = sb[j] - mu[j] * sa[j];
   }
+  if (EXTRA) lane_group_pairs<A, VEC>(p, l, sm_c1, sm_c2, c1, c2);
 }
 
 // ---------------------------------------------------------------------------------------------
