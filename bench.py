@@ -66,6 +66,11 @@ def parse_args():
     ap.add_argument("--switch-cost", action="store_true",
                     help="no headline: event-timed duration of each kernel of the workload when it follows itself and when it "
                          "follows a different kernel whose data is tiny (a 1 MB plain copy; a small GroupNorm forward)")
+    ap.add_argument("--code-placement", action="store_true",
+                    help="no headline: per-kernel times of the workload (event-timed inside the sweep) in four child processes that "
+                         "first load 0, 1, 2, 3 copies of the library under other names, which moves the code of the library proper "
+                         "by one 2 MB slot each: how much of a kernel's time depends on where the loader put its code")
+    ap.add_argument("--code-placement-child", type=int, default=-1, help=argparse.SUPPRESS)
     ap.add_argument("--counter-workload", action="store_true",
                     help="no timing: one 256 MiB plain copy (calibration) and a few fwd+bwd calls per shape, for a rocprofv3 --pmc run")
     return ap.parse_args()
@@ -480,6 +485,50 @@ def switch_cost(names, device):
         torch.cuda.empty_cache()
 
 
+def code_placement_child(names, device, copies):
+    """One process of --code-placement: load `copies` copies of the library first (each one's first kernel launch makes the
+    runtime load a code object, which takes the next 2 MB-aligned slot), then time the workload's kernels inside the sweep."""
+    import ctypes
+    import shutil
+    import tempfile
+    import torch
+    from gnnhwc import _cabi
+    import workloads as configs
+
+    keep = []
+    tmp = tempfile.mkdtemp(prefix="gnnhwc_copies_")
+    a = torch.empty((1 << 16,), dtype=torch.uint8, device=device)
+    b = torch.empty_like(a)
+    for i in range(copies):
+        dst = os.path.join(tmp, "libcopy%d.so" % i)
+        shutil.copy(_cabi.LIB_PATH, dst)
+        lib = ctypes.CDLL(dst)
+        lib.gnnhwc_debug_copy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+        lib.gnnhwc_debug_copy(b.data_ptr(), a.data_ptr(), a.numel(), None)
+        torch.cuda.synchronize()
+        keep.append(lib)
+    probs = [Problem(configs.CONFIGS[n], device) for n in names]
+    r = kernel_profile(probs, 100)
+    cells = []
+    for n in names:
+        for kind, (us, per_call) in sorted(r[n].items()):
+            cells.append("%s %s %.2f" % (n, kind, us))
+    print("copies loaded first: %d | %s | sum %.2f" % (copies, " | ".join(cells),
+                                                        sum(us * pc for k in r.values() for us, pc in k.values())))
+    shutil.rmtree(tmp, ignore_errors=True)
+
+
+def code_placement(workload):
+    import subprocess
+    print("# event-timed microseconds per launch inside the sweep; one child process per line")
+    for copies in (0, 1, 2, 3, 0, 1):
+        out = subprocess.run([sys.executable, os.path.abspath(__file__), "--workload", workload, "--code-placement-child", str(copies)],
+                             capture_output=True, text=True)
+        lines = [ln for ln in out.stdout.splitlines() if ln.startswith("copies loaded first")]
+        print(lines[-1] if lines else "child failed: " + out.stderr.strip().splitlines()[-1])
+        sys.stdout.flush()
+
+
 def cpu_baseline(cfg_names, seconds):
     """torch's CPU GroupNorm + activation + autograd on the host cores, same seeded tensors and dtype."""
     import torch
@@ -721,6 +770,9 @@ def main():
         print("bench.py: this build measures one GPU only (GroupNorm statistics are per sample; nothing is exchanged "
               "between GPUs). Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
+    if args.code_placement:  # (the children touch the GPU; this process does not)
+        code_placement(args.workload)
+        return
     if args.timeline:
         os.environ["GNNHWC_TRACE"] = "2"  # read by the library at its first single-launch call
     import torch
@@ -732,6 +784,10 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
     use_graph = args.graph
+    if args.code_placement_child >= 0:
+        code_placement_child(list(configs.SD_UNET_SWEEP) if args.workload == "sd_unet" else [args.workload], device,
+                             args.code_placement_child)
+        return
     if args.switch_cost:
         switch_cost(list(configs.SD_UNET_SWEEP) if args.workload == "sd_unet" else
                     list(configs.ALL_NAMES) if args.workload == "all" else [args.workload], device)
