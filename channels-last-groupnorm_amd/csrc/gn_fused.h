@@ -45,7 +45,7 @@ struct SyncArea {
   unsigned crec_bytes;
   void *frecs;                // 16-byte records {value0, value1, epoch} per (sample, group): results of the second level
   unsigned frec_bytes;        // (two_level != 0 only)
-  int two_level;              // the groups' tile records are merged once, by one workgroup per group, not by every workgroup
+  int two_level;              // host side only: selects the TWO_LEVEL instantiation of the kernel
   unsigned long long epoch;   // value that marks "written in this call"
   const unsigned long long *generation;  // device counter that replaces the epoch in captured launches (resident_epoch)
   unsigned long long *status; // set to the epoch if a wait of this call timed out
@@ -241,7 +241,10 @@ constexpr int kAddNone = 0, kAddChannel = 1, kAddResidual = 2;
 constexpr int fused_fwd_waves(int nv, int add) {
   return add == kAddResidual ? (nv <= 4 ? 4 : nv <= 8 ? 3 : nv <= 16 ? 2 : 1) : (nv <= 8 ? 4 : nv <= 16 ? 3 : 2);
 }
-template <typename T, typename PT, int VEC, int ACT, int NV, int ADD>
+// TWO_LEVEL: the exchange of a launch with many row tiles per sample (two_level_exchange on the host).  A template
+// parameter, not a run-time switch: the code of the form a launch does not use would sit in the middle of the path every
+// workgroup executes once, and these kernels are sensitive to their own size.
+template <typename T, typename PT, int VEC, int ACT, int NV, int ADD, bool TWO_LEVEL>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fwd_waves(NV, ADD)))) void fused_fwd_kernel(
     const T *__restrict__ x, T *__restrict__ y, SyncArea sync_arg, const void *w, const void *b, void *mean_out,
     void *rstd_out, int sdtype, int ydtype, acc_t<T> eps, AddArgs add, Plan p) {
@@ -372,7 +375,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
     record_store(rb, record_slot(q, p.G, (int)n, l.tile, l.chunk, g), mu, s2, sync.epoch);
   });
   trace_point(sync, 2);
-  if (sync.two_level) {
+  if constexpr (TWO_LEVEL) {
     // second level: the groups this workgroup owns, one at a time with all 256 lanes (usually one group or none)
     const __amdgpu_buffer_rsrc_t fb = final_record_buffer(sync);
     const A total = (A)p.D * (A)p.R;
@@ -483,7 +486,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
 //   group records   : {A, B, epoch} per (n, chunk, group, tile) of this launch
 //   channel records : {S1, S2, epoch} per (n, tile, channel) of the whole tensor (they feed dgamma / dbeta)
 // ---------------------------------------------------------------------------------------------
-template <typename T, typename PT, int VEC, int ACT, int NV>
+template <typename T, typename PT, int VEC, int ACT, int NV, bool TWO_LEVEL>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 ? 4 : NV <= 8 ? 3 : NV <= 22 ? 2 : 1))) void fused_bwd_kernel(
     const T *__restrict__ x, const T *__restrict__ dy, T *__restrict__ dx, const void *mean, const void *rstd, int sdtype,
     const void *w, const void *b, SyncArea sync_arg, void *dw, void *db, const void *mean_all, const void *rstd_all,
@@ -607,7 +610,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
   }
   __syncthreads();
   trace_point(sync, 2);
-  if (sync.two_level) {
+  if constexpr (TWO_LEVEL) {
     // second level (see owns_group): the groups this workgroup owns, one at a time with all 256 lanes
     const __amdgpu_buffer_rsrc_t fb = final_record_buffer(sync);
     __shared__ A sm_x[8];

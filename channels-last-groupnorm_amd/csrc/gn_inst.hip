@@ -1,6 +1,8 @@
 // Kernel instantiations and launch sequences for ONE element type, selected with -DGN_INST_DTYPE=0..3
 // (f32, f64, f16, bf16).  Built four times so the four types compile in parallel.
 #include "gn_host.h"
+#include <algorithm>
+
 #include "gn_fused.h"
 #include "gn_kernels.h"
 
@@ -166,8 +168,9 @@ size_t stat_size(int sdtype) { return sdtype == GN_F32 ? 4 : sdtype == GN_F64 ? 
 // One NV variant, the tensor cut into `batches` launches over consecutive samples (1: the whole tensor).
 template <typename PT, int ACT, int NV, int ADD> bool try_resident_fwd_nv(const FwdArgs &a, int batches) {
   if (NV < resident_min_rows()) return false;
-  auto kernel = fused_fwd_kernel<elem_t, PT, kVec, ACT, NV, ADD>;
-  static const int slots = resident_slots(kernel);
+  auto kernel_all = fused_fwd_kernel<elem_t, PT, kVec, ACT, NV, ADD, false>;  // every workgroup polls every tile
+  auto kernel_two = fused_fwd_kernel<elem_t, PT, kVec, ACT, NV, ADD, true>;   // two-level exchange (many tiles)
+  static const int slots = std::min(resident_slots(kernel_all), resident_slots(kernel_two));
   const int64_t per = (a.plan.N + batches - 1) / batches;
   Plan p;
   if (!resident_tiling(a.plan, per, NV, slots, p)) return false;
@@ -186,7 +189,8 @@ template <typename PT, int ACT, int NV, int ADD> bool try_resident_fwd_nv(const 
     if (add.residual) add.residual = (const elem_t *)add.residual + n0 * sample;
     if (add.sum_out) add.sum_out = (elem_t *)add.sum_out + n0 * sample;
     if (add.channel_bias) add.channel_bias = (const char *)add.channel_bias + n0 * a.plan.C * stat_size(add.channel_bias_dtype);
-    launch(ADD != kAddNone ? kKindFusedFwdAdd : kKindFusedFwd, kernel, tile_grid(pb, 0), dim3(kBlock), a.stream,
+    launch(ADD != kAddNone ? kKindFusedFwdAdd : kKindFusedFwd, r.sync.two_level ? kernel_two : kernel_all, tile_grid(pb, 0),
+           dim3(kBlock), a.stream,
            (const elem_t *)a.x + n0 * sample, (elem_t *)((char *)a.y + n0 * sample * stat_size(a.ydtype)), r.sync, a.w, a.b,
            a.mean ? (char *)a.mean + n0 * a.plan.G * stat_size(a.sdtype) : nullptr,
            a.rstd ? (char *)a.rstd + n0 * a.plan.G * stat_size(a.sdtype) : nullptr, a.sdtype, a.ydtype, (A)a.eps, add, pb);
@@ -242,8 +246,9 @@ bool try_resident_fwd(const FwdArgs &a) {
 #if GN_PART_BWD
 template <typename PT, int ACT, int NV> bool try_resident_bwd_nv(const BwdArgs &a, int batches) {
   if (NV < resident_min_rows()) return false;
-  auto kernel = fused_bwd_kernel<elem_t, PT, kVec, ACT, NV>;
-  static const int slots = resident_slots(kernel);
+  auto kernel_all = fused_bwd_kernel<elem_t, PT, kVec, ACT, NV, false>;
+  auto kernel_two = fused_bwd_kernel<elem_t, PT, kVec, ACT, NV, true>;
+  static const int slots = std::min(resident_slots(kernel_all), resident_slots(kernel_two));
   const int64_t per = (a.plan.N + batches - 1) / batches;
   Plan p;
   if (!resident_tiling(a.plan, per, NV, slots, p)) return false;
@@ -264,7 +269,8 @@ template <typename PT, int ACT, int NV> bool try_resident_bwd_nv(const BwdArgs &
     ResidentWorkspace r = resident_bwd_ws(a.ws, pb);
     arm_generation(r, cap);
     const bool last = n0 + per >= a.plan.N;
-    launch(kKindFusedBwd, kernel, tile_grid(pb, 0), dim3(kBlock), a.stream, (const elem_t *)a.x + n0 * sample,
+    launch(kKindFusedBwd, r.sync.two_level ? kernel_two : kernel_all, tile_grid(pb, 0), dim3(kBlock), a.stream,
+           (const elem_t *)a.x + n0 * sample,
            (const elem_t *)a.dy + n0 * sample, (elem_t *)a.dx + n0 * sample, (const char *)a.mean + n0 * a.plan.G * ssz,
            (const char *)a.rstd + n0 * a.plan.G * ssz, a.sdtype, a.w, a.b, r.sync, last ? a.dw : nullptr,
            last ? a.db : nullptr, a.mean, a.rstd, n0, a.plan.N, pb);
