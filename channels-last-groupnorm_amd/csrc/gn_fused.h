@@ -486,8 +486,15 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
 //   group records   : {A, B, epoch} per (n, chunk, group, tile) of this launch
 //   channel records : {S1, S2, epoch} per (n, tile, channel) of the whole tensor (they feed dgamma / dbeta)
 // ---------------------------------------------------------------------------------------------
-template <typename T, typename PT, int VEC, int ACT, int NV, bool TWO_LEVEL>
-__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 ? 4 : NV <= 8 ? 3 : NV <= 22 ? 2 : 1))) void fused_bwd_kernel(
+// XW: 0 keeps the tile of x in registers next to the tile of g' (NV rows each).  XW > 0 keeps g' only and streams x
+// through a window of XW rows, twice: once for the sums and once, in the opposite direction (so that the window's
+// last rows serve both passes), for dx.  That form holds a tensor half again as large at the price of reading
+// (NV - XW) / NV of x a second time: 4 - XW / NV tensors of traffic, against the 5 of the multi-launch backward.
+constexpr int fused_bwd_waves(int nv, int xw) {
+  return xw > 0 ? (nv <= 24 ? 3 : 2) : (nv <= 4 ? 4 : nv <= 8 ? 3 : nv <= 22 ? 2 : 1);
+}
+template <typename T, typename PT, int VEC, int ACT, int NV, bool TWO_LEVEL, int XW = 0>
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bwd_waves(NV, XW)))) void fused_bwd_kernel(
     const T *__restrict__ x, const T *__restrict__ dy, T *__restrict__ dx, const void *mean, const void *rstd, int sdtype,
     const void *w, const void *b, SyncArea sync_arg, void *dw, void *db, const void *mean_all, const void *rstd_all,
     int64_t n0, int64_t n_all, Plan p) {
@@ -508,7 +515,28 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
   const SafeLane sfl = safe_lane<VEC>(p, l, n);
   const int64_t off = sfl.off;
   const int64_t step = (int64_t)p.rpi * p.C;
-  typename LV::raw_t bx[NV], bd[NV];
+  constexpr int NX = XW > 0 ? XW : NV;  // rows of x held at a time; row u lives in bx[u % NX]
+  static_assert(XW >= 0 && XW <= NV, "window within the tile");
+  typename LV::raw_t bx[NX], bd[NV];
+  auto row_offset = [&](int u) { return off + (int64_t)clamp_row(u, sfl.rows) * step; };
+  // XW > 0: rows are requested all through the kernel, so their addresses must be cheap to form again: the tile's
+  // (uniform) base plus a 32-bit byte offset per lane and row (the host admits only tiles below 2 GiB)
+  const int64_t tile_base = (n * p.R + l.row0) * p.C;
+  const unsigned lane_byte0 = (unsigned)(((sfl.live ? l.ty : 0) * p.C + sfl.c) * (int)sizeof(T));
+  const unsigned step_bytes = (unsigned)(p.rpi * p.C * (int)sizeof(T));
+  // (every pass forms them from its own opaque copy of the three terms: offsets kept from one pass for the next
+  // would cost a register per row)
+  struct RowTerms { unsigned lane0, step; int rows; };
+  auto fresh_terms = [&]() {
+    RowTerms t{lane_byte0, step_bytes, sfl.rows};
+    pin(t.lane0);
+    pin(t.step);
+    pin(t.rows);
+    return t;
+  };
+  auto tile_row = [&](const T *base, const RowTerms &t, int u) {
+    return (const T *)((const char *)(base + tile_base) + (t.lane0 + (unsigned)clamp_row(u, t.rows) * t.step));
+  };
   trace_point(sync, 0);
   // the small loads go first: loads return in order, so the statistics and parameters, which the first row's
   // arithmetic needs, must not queue behind the whole tile.  Nothing here is under a branch (idle lanes read valid
@@ -526,11 +554,20 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
     gamma0 = w ? gv : (A)1;
   }
   issue_order_fence();
+  if constexpr (XW == 0) {
 #pragma unroll
-  for (int u = 0; u < NV; ++u) {
-    const int64_t o = off + (int64_t)clamp_row(u, sfl.rows) * step;
-    bx[u] = LV::load(x + o);
-    bd[u] = LV::load(dy + o);
+    for (int u = 0; u < NV; ++u) {
+      const int64_t o = row_offset(u);
+      bx[u] = LV::load(x + o);
+      bd[u] = LV::load(dy + o);
+    }
+  } else {
+    // the window of x first (row 0's arithmetic needs it), then all of dy; the rest of x follows row by row below
+    const RowTerms t0 = fresh_terms();
+#pragma unroll
+    for (int u = 0; u < XW; ++u) bx[u] = LV::load(tile_row(x, t0, u));
+#pragma unroll
+    for (int u = 0; u < NV; ++u) bd[u] = LV::load(tile_row(dy, t0, u));
   }
   commit_chunk_stats<A>(st, l, sm_mu, sm_rs);
   __builtin_amdgcn_s_setprio(2);  // towards the exchange: ahead of wavefronts that are already past theirs
@@ -552,21 +589,42 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
         for (int u = 0; u < NV; ++u)
           if (u >= rows) bd[u] = zero;
       }
+      const RowTerms t1 = fresh_terms();
 #pragma unroll
       for (int u = 0; u < NV; ++u) {
         A vx[VEC], vd[VEC];
-        pin(bx[u]);  // one row at a time: cheap activations otherwise tempt the scheduler into unpacking many
-        pin(bd[u]);  // rows ahead, which costs more registers than the tile itself
-        LV::unpack(bx[u], vx);
+        pin(bx[u % NX]);  // one row at a time: cheap activations otherwise tempt the scheduler into unpacking many
+        pin(bd[u]);       // rows ahead, which costs more registers than the tile itself
+        LV::unpack(bx[u % NX], vx);
         LV::unpack(bd[u], vd);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) {
+          if constexpr (XW > 0 && VEC >= 4) {
+            // half a row at a time: the temporaries of a costly derivative for a whole row do not fit beside the tile
+            if (j == VEC / 2) {
+#pragma unroll
+              for (int i = 0; i < VEC / 2; ++i) { pin(vd[i]); pin(s1[i]); pin(s2[i]); }
+#pragma unroll
+              for (int i = VEC / 2; i < VEC; ++i) { pin(vx[i]); pin(vd[i]); }
+            }
+          }
           const A g = vd[j] * act_bwd<ACT, A>(vx[j] * sa[j] + sb[j]);
           s1[j] += g * vx[j];
           s2[j] += g;
           vd[j] = g;
         }
         bd[u] = LV::pack(vd);
+        if constexpr (XW > 0) {
+          // the sums are brought up to date row by row: left alone, the scheduler postpones the chains of the window's
+          // last rows to the end and keeps their unpacked g' alive until then
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) { pin(s1[j]); pin(s2[j]); }
+          pin(bd[u]);  // packed here and now (the conversion otherwise sinks towards the dx phase, g' staying unpacked)
+          if (u + XW < NV) {
+            issue_order_fence();  // not before the rows ahead of it are consumed: the slot is the register budget
+            bx[u % NX] = LV::load(tile_row(x, t1, u + XW));  // the slot's next row
+          }
+        }
       }
     }
     trace_point(sync, 6, (float)(s1[0] + s2[0]));
@@ -694,16 +752,38 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NV <= 4 
   trace_point(sync, 3);
   if (rows > 0) {
     lane_group_pairs<A, VEC>(p, l, sm1, sm2, c1, c2);
+    if constexpr (XW == 0) {
 #pragma unroll
-    for (int u = 0; u < NV; ++u) {
-      if (u < rows) {
+      for (int u = 0; u < NV; ++u) {
+        if (u < rows) {
+          A vx[VEC], vd[VEC];
+          pin(bx[u]);
+          LV::unpack(bx[u], vx);
+          LV::unpack(bd[u], vd);  // g'
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) vd[j] = sa[j] * vd[j] + (c1[j] * vx[j] + c2[j]);
+          store_streaming<LV>(dx + off + (int64_t)u * step, LV::pack(vd));
+        }
+      }
+    } else {
+      // from the last row down: the window still holds rows NV - XW ... NV - 1 of the first pass, and every slot is
+      // refilled with the row XW above as soon as its row is done (unconditionally: the waits count loads exactly)
+      const RowTerms t2 = fresh_terms();
+#pragma unroll
+      for (int k = 0; k < NV; ++k) {
+        const int u = NV - 1 - k;
         A vx[VEC], vd[VEC];
-        pin(bx[u]);
-        LV::unpack(bx[u], vx);
+        pin(bx[u % NX]);
+        pin(bd[u]);
+        LV::unpack(bx[u % NX], vx);
         LV::unpack(bd[u], vd);  // g'
 #pragma unroll
         for (int j = 0; j < VEC; ++j) vd[j] = sa[j] * vd[j] + (c1[j] * vx[j] + c2[j]);
-        store_streaming<LV>(dx + off + (int64_t)u * step, LV::pack(vd));
+        if (u < rows) store_streaming<LV>((T *)tile_row(dx, t2, u), LV::pack(vd));
+        if (u >= XW) {
+          issue_order_fence();
+          bx[u % NX] = LV::load(tile_row(x, t2, u - XW));
+        }
       }
     }
   }

@@ -244,14 +244,16 @@ bool try_resident_fwd(const FwdArgs &a) {
 #endif  // !GN_PART_BWD
 
 #if GN_PART_BWD
-template <typename PT, int ACT, int NV> bool try_resident_bwd_nv(const BwdArgs &a, int batches) {
+template <typename PT, int ACT, int NV, int XW = 0> bool try_resident_bwd_nv(const BwdArgs &a, int batches) {
   if (NV < resident_min_rows()) return false;
-  auto kernel_all = fused_bwd_kernel<elem_t, PT, kVec, ACT, NV, false>;
-  auto kernel_two = fused_bwd_kernel<elem_t, PT, kVec, ACT, NV, true>;
+  auto kernel_all = fused_bwd_kernel<elem_t, PT, kVec, ACT, NV, false, XW>;
+  auto kernel_two = fused_bwd_kernel<elem_t, PT, kVec, ACT, NV, true, XW>;
   static const int slots = std::min(resident_slots(kernel_all), resident_slots(kernel_two));
   const int64_t per = (a.plan.N + batches - 1) / batches;
   Plan p;
   if (!resident_tiling(a.plan, per, NV, slots, p)) return false;
+  // (the windowed form addresses the rows of a tile by 32-bit byte offsets from the tile's first row)
+  if (XW > 0 && (int64_t)p.tile_rows * p.C * (int64_t)sizeof(elem_t) >= ((int64_t)1 << 31)) return false;
   // the channel records of every sample stay in the workspace until the last launch has summed them
   const size_t crec_need = (size_t)a.plan.N * p.tiles * a.plan.C * 16;
   if (crec_need > resident_crec_bytes((int64_t)p.lpr * p.vec)) return false;
@@ -279,11 +281,15 @@ template <typename PT, int ACT, int NV> bool try_resident_bwd_nv(const BwdArgs &
 }
 template <typename PT, int ACT> bool try_resident_bwd_act(const BwdArgs &a) {
   const int most = a.plan.N < worthwhile_batches(a.plan, true) ? (int)a.plan.N : worthwhile_batches(a.plan, true);
-  for (int b = 1; b <= most; ++b)
+  for (int b = 1; b <= most; ++b) {
     if (try_resident_bwd_nv<PT, ACT, 4>(a, b) || try_resident_bwd_nv<PT, ACT, 8>(a, b) ||
         try_resident_bwd_nv<PT, ACT, 16>(a, b) || try_resident_bwd_nv<PT, ACT, 22>(a, b) ||
         try_resident_bwd_nv<PT, ACT, 32>(a, b))
       return true;
+    // too large for two tiles in registers: the form that keeps g' and reads most of x twice, before the tensor is cut
+    // into more launches (measured on bf16 (N, 320, 128, 128): 33.7 against 39.3 us at N = 5, 38.6 against 43.4 at N = 6)
+    if (try_resident_bwd_nv<PT, ACT, 32, 12>(a, b) || try_resident_bwd_nv<PT, ACT, 36, 8>(a, b)) return true;
+  }
   return false;
 }
 template <typename PT> bool try_resident_bwd_pt(const BwdArgs &a) {

@@ -14,6 +14,7 @@ import torch
 
 from oracle import gn_oracle as orc
 from tests import configs
+from gnnhwc import _cabi
 from tests.gpu_harness import as_np64, cabi_bwd, cabi_fwd, err, nrc_view
 
 pytestmark = pytest.mark.gpu
@@ -119,6 +120,41 @@ def test_random_medium_shapes(family, N, R, C, G, act, dtype, device):
     torch's own GroupNorm + activation + autograd in float64 on the device (the results contract; the C oracle would
     need minutes for these sizes); bars as for the configurations."""
     print("medium", family, N, R, C, G, act, dtype, flush=True)
+    _check_against_torch(N, R, C, G, act, dtype, device)
+
+
+# One sample of 47 - 75 MB: too large for the single-launch backward that keeps x and g' in registers, within reach of
+# the one that keeps g' and streams x through a window twice.  Rows that do not fill the last tile, groups that
+# straddle the 64-channel chunks, every activation, the three 4-byte-accumulated types.
+LARGE_BACKWARD_SHAPES = [
+    (1, 150037, 192, 24, "silu", torch.bfloat16),
+    (1, 40003, 320, 32, "relu", torch.float32),
+    (1, 512 * 512 - 511, 128, 32, "gelu", torch.float16),
+    (1, 9001, 3200, 32, "gelu_tanh", torch.bfloat16),
+    (1, 100000, 160, 1, "identity", torch.float32),
+]
+
+
+@pytest.mark.parametrize("N,R,C,G,act,dtype", LARGE_BACKWARD_SHAPES)
+def test_large_single_sample_backward(family, N, R, C, G, act, dtype, device):
+    """The windowed single-launch backward against torch in float64 (bars as for the configurations), and that it is
+    the kernel that ran: one launch of the single-launch backward, none of the multi-launch kernels."""
+    print("large backward", family, N, R, C, G, act, dtype, flush=True)
+    _cabi.profile_collect()
+    _cabi.profile_enable(True)
+    try:
+        _check_against_torch(N, R, C, G, act, dtype, device)
+    finally:
+        _cabi.profile_enable(False)
+    launches = {k: v[0] for k, v in _cabi.profile_collect().items() if v[0]}
+    print(launches, flush=True)
+    if family == "resident":
+        assert launches.get("fused_bwd") == 1 and "bwd_reduce" not in launches and "bwd_dx" not in launches, launches
+    else:
+        assert launches.get("bwd_dx") == 1 and "fused_bwd" not in launches, launches
+
+
+def _check_against_torch(N, R, C, G, act, dtype, device):
     gen = torch.Generator().manual_seed(N * 1000003 + R * 101 + C)
     x = (torch.randn((N, R, C), generator=gen) * 1.7 + torch.randn((C,), generator=gen)).to(dtype).to(device)
     dy = torch.randn((N, R, C), generator=gen).to(dtype).to(device)
