@@ -287,7 +287,7 @@ template <typename PT, int ACT> bool try_resident_bwd_act(const BwdArgs &a) {
         try_resident_bwd_nv<PT, ACT, 32>(a, b))
       return true;
     // too large for two tiles in registers: the form that keeps g' and reads most of x twice, before the tensor is cut
-    // into more launches (measured on bf16 (N, 320, 128, 128): 33.7 against 39.3 us at N = 5, 38.6 against 43.4 at N = 6)
+    // into more launches (measured on bf16 (N, 320, 128, 128): 32.6 against 39.3 us at N = 5, 37.2 against 43.4 at N = 6)
     // (window: what the registers leave beside 32 rows of g', 16 rows for 16-bit data)
     constexpr int window = sizeof(elem_t) == 2 ? 16 : 12;
     if (try_resident_bwd_nv<PT, ACT, 32, window>(a, b) || try_resident_bwd_nv<PT, ACT, 36, 8>(a, b)) return true;
