@@ -310,6 +310,28 @@ BWD_STAMPS = ((0, "workgroup starts"), (1, "mean / rstd staged"), (6, "tile sums
               (5, "dgamma / dbeta written (workgroups of sample 0)"))
 
 
+ARRIVAL_STAMP = {"fwd": 1, "bwd": 6}  # the stamp taken when all rows of the tile are in registers
+
+
+def arrival_by_dispatch_order(t, which, cus=256):
+    """Median 'rows arrived' time of the workgroups of one traced launch (stamps `t`, one row per workgroup in the
+    order of their linear block index, which is the order they are dispatched in), grouped by cus: the first `cus`
+    workgroups are the first on their CU, the next `cus` the second, and so on."""
+    import numpy as np
+
+    pt = ARRIVAL_STAMP[which]
+    rel = (t[:, pt] - t[:, 0].min()) / 100.0
+    return [float(np.median(rel[i:i + cus])) for i in range(0, t.shape[0], cus)]
+
+
+def print_arrival_by_dispatch_order(rows_by_rep):
+    if not rows_by_rep or len(rows_by_rep[0]) < 2:
+        return
+    n = min(len(r) for r in rows_by_rep)
+    med = [statistics.median(r[i] for r in rows_by_rep) for i in range(n)]
+    print("    %-58s %s" % ("  all rows arrived, workgroups 0-255 / 256-511 / ... (median)", " / ".join("%7.2f" % m for m in med)))
+
+
 def timeline(names, device, reps=5):
     """In-kernel timeline of the single-launch kernels.  Thread 0 of every workgroup stamps a 100 MHz wall clock at its
     phase boundaries (GNNHWC_TRACE=2: the stamps do not wait for outstanding memory operations, so the kernel overlaps
@@ -348,6 +370,7 @@ def timeline(names, device, reps=5):
             torch.cuda.synchronize()
             time.sleep(0.002)
             rows = []
+            waves = []
             for _ in range(reps):
                 p.step(0, stream, "both")  # the traced launch runs behind other kernels, as in the sweep: a backward behind its
                 if which == "fwd":         # own forward, a forward behind the backward of the call before
@@ -357,6 +380,7 @@ def timeline(names, device, reps=5):
                 t = words.astype(np.int64)
                 live = t[:, 0] >= t[:, 0].max() - 300  # started within 3 us of the latest start: the workgroups of this launch
                 t = t[live]
+                waves.append(arrival_by_dispatch_order(t, which))
                 rel = (t - t[:, 0].min()) / 100.0
                 taken = {}
                 for pt, _ in stamps:  # a stamp older than the launch was not taken by this launch (stamp 5: sample 0 only)
@@ -373,6 +397,8 @@ def timeline(names, device, reps=5):
                     continue
                 med = [statistics.median(v[i] for v in vals) for i in range(3)]
                 print("    %-58s %7.2f / %7.2f / %7.2f" % (label, med[0], med[1], med[2]))
+                if pt == ARRIVAL_STAMP[which]:
+                    print_arrival_by_dispatch_order(waves)
         del p
         torch.cuda.empty_cache()
 
@@ -402,6 +428,7 @@ def timeline_in_sweep(names, device, reps=5):
                   % (p.cfg.name, which, ", ".join("%s %.2f us" % kv for kv in evs.items() if not kv[0].startswith("fused"))))
             continue
         rows = []
+        waves = []
         for _ in range(reps):
             torch.cuda.synchronize()
             time.sleep(0.002)
@@ -415,6 +442,7 @@ def timeline_in_sweep(names, device, reps=5):
             t = words.astype(np.int64)
             live = t[:, 0] >= t[:, 0].max() - 300
             t = t[live]
+            waves.append(arrival_by_dispatch_order(t, which))
             rel = (t - t[:, 0].min()) / 100.0
             taken = {}
             for pt, _ in stamps:
@@ -430,6 +458,8 @@ def timeline_in_sweep(names, device, reps=5):
                 continue
             med = [statistics.median(v[i] for v in vals) for i in range(3)]
             print("    %-58s %7.2f / %7.2f / %7.2f" % (label, med[0], med[1], med[2]))
+            if pt == ARRIVAL_STAMP[which]:
+                print_arrival_by_dispatch_order(waves)
 
 
 def switch_cost(names, device):
