@@ -767,7 +767,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
       }
     } else {
       // from the last row down: the window still holds rows NV - XW ... NV - 1 of the first pass, and every slot is
-      // refilled with the row XW above as soon as its row is done (unconditionally: the waits count loads exactly)
+      // refilled with the row XW below it as soon as its row is done (unconditionally: the waits count loads exactly)
       const RowTerms t2 = fresh_terms();
 #pragma unroll
       for (int k = 0; k < NV; ++k) {
