@@ -358,8 +358,8 @@ unsigned long long *trace_buffer() {
   }();
   return buf;
 }
-// Host-pinned, device-visible word that a single-launch kernel sets when one of its bounded waits expires
-// (its workgroups were not all resident at once, so its output is wrong).  The next API call reports it.
+// Host-pinned, device-visible word that a single-launch kernel sets when one of its bounded waits expires (its
+// workgroups were not all resident at once, and it recomputed the records it was waiting for): gnnhwc_resident_status.
 unsigned long long *resident_status() {
   static unsigned long long *word = []() -> unsigned long long * {
     // the first call may come while the thread is capturing a graph: allocation is legal there in relaxed mode
@@ -383,10 +383,17 @@ int resident_min_rows() {
   static const int v = env_int("GNNHWC_RESIDENT_MIN_ROWS", 0);
   return v;
 }
-constexpr int kDefaultSpinLimit = 1 << 20;  // polls per wait; a poll is a device-scope round trip, about a microsecond
+// Polls per wait.  A poll is a device-scope round trip and a short sleep, about a microsecond, so a lane waits about a
+// millisecond for workgroups that are not resident yet before it recomputes their records itself -- which costs a few
+// milliseconds per launch: waiting about as long as the recovery takes, and no longer.
+constexpr int kDefaultSpinLimit = 1 << 10;
 std::atomic<int> g_spin_limit{kDefaultSpinLimit};
 int resident_spin_limit() { return g_spin_limit.load(std::memory_order_relaxed); }
 
+bool cooperative_launches() {
+  static const bool v = env_int("GNNHWC_COOPERATIVE", 0) != 0;
+  return v;
+}
 std::atomic<int> g_resident{-1};  // -1: follow the environment
 bool resident_enabled() {
   static const int off = env_int("GNNHWC_DISABLE_RESIDENT", 0);
@@ -411,18 +418,14 @@ bool profile_events(int kind, hipEvent_t *start, hipEvent_t *stop) {
 
 using namespace gn;
 
-// A timed-out single-launch kernel leaves wrong output behind: say so on the next call (nothing is launched by
-// that call), and use the streaming kernels for the rest of the process.
-static int check_resident_health() {
-  if (!g_status_live.load(std::memory_order_relaxed)) return GNNHWC_OK;
+// A single-launch kernel some of whose waits expired has recomputed what it was waiting for: its results are right, it
+// only took longer.  The status word records that it happened; reading clears it.
+static int degraded_since_last_query() {
+  if (!g_status_live.load(std::memory_order_relaxed)) return 0;
   volatile unsigned long long *w = resident_status();
-  if (!w || *w == 0) return GNNHWC_OK;
+  if (!w || *w == 0) return 0;
   *w = 0;
-  g_resident.store(0, std::memory_order_relaxed);
-  return fail(GNNHWC_ERR_LAUNCH,
-              "an earlier single-launch GroupNorm kernel could not synchronise its workgroups (they were not all resident "
-              "at once, e.g. because another stream was using the device); the results of that call are invalid. "
-              "The multi-launch kernels are used from now on");
+  return 1;
 }
 
 // ---- forward that allocates nothing -------------------------------------------------------------------------
@@ -497,8 +500,6 @@ static int forward(const void *x, const AddArgs &add, const void *weight, const 
     return fail(GNNHWC_ERR_INVALID_ARGUMENT, "y_dtype %d with dtype %d: y is written in dtype, or as F16 / BF16 for F32 data",
                 y_dtype, dtype);
   if (N == 0 || R == 0) return GNNHWC_OK;  // nothing to normalise; mean / rstd of an empty slab are left untouched
-  rc = check_resident_health();
-  if (rc != GNNHWC_OK) return rc;
   if (!x || !y) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "x and y must not be null");
   if (y_dtype != dtype && y == x) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "y of another type than x cannot replace x in place");
   const size_t need = streaming_only ? align_up(fwd_ws_bytes(N, R, C, G, dtype, true), 256) : gnnhwc_fwd_workspace_bytes(N, R, C, G, dtype);
@@ -605,8 +606,6 @@ int gnnhwc_bwd(const void *dy, const void *x, const void *weight, const void *bi
     if (e0 != hipSuccess) return fail(GNNHWC_ERR_LAUNCH, "backward launch failed: %s", hipGetErrorString(e0));
     return GNNHWC_OK;
   }
-  rc = check_resident_health();
-  if (rc != GNNHWC_OK) return rc;
   if (!dy || !x || !mean || !rstd || !dx)
     return fail(GNNHWC_ERR_INVALID_ARGUMENT, "dy, x, mean, rstd and dx must not be null");
   const size_t need = gnnhwc_bwd_workspace_bytes(N, R, C, G, dtype);
@@ -660,7 +659,7 @@ int gnnhwc_profile_collect(int64_t *launches, double *total_ms) {
   return rc;
 }
 
-int gnnhwc_resident_status(void) { return check_resident_health(); }
+int gnnhwc_resident_status(void) { return degraded_since_last_query(); }
 
 int gnnhwc_set_resident(int on) {
   const int before = resident_enabled() ? 1 : 0;
@@ -669,7 +668,7 @@ int gnnhwc_set_resident(int on) {
 }
 
 int gnnhwc_debug_set_spin_limit(int polls) {
-  if (polls < 0 && polls != -2) polls = kDefaultSpinLimit;  // -2: every wait gives up at its first poll, ready or not
+  if (polls < 0 && polls != -2) polls = kDefaultSpinLimit;  // -2: every wait takes the recovery path at once, ready or not
   return g_spin_limit.exchange(polls, std::memory_order_relaxed);
 }
 
@@ -711,8 +710,6 @@ size_t gnnhwc_nchw_workspace_bytes(int64_t N, int64_t C, int64_t R, int64_t G, i
   return align_up(nchw_workspace_elems(N, C, R, 1, backward != 0) * acc_size(dtype), 256);
 }
 static int nchw_call(NchwArgs &a, int dtype, void *workspace, size_t workspace_bytes, const char *what) {
-  const int health = check_resident_health();  // an earlier single-launch call of the process may have failed
-  if (health != GNNHWC_OK) return health;
   const size_t need = gnnhwc_nchw_workspace_bytes(a.N, a.C, a.R, a.G, dtype, a.backward ? 1 : 0);
   if (!workspace || !aligned16(workspace) || workspace_bytes < need)
     return fail(GNNHWC_ERR_WORKSPACE, "%s workspace must be 16-byte aligned and at least %zu bytes (got %p, %zu bytes)", what,

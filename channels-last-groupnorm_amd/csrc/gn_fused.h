@@ -25,26 +25,40 @@
 //    that owns it).  The instruction set does not promise it in writing; if it did not hold, a consumer could pair a
 //    fresh epoch with stale values.  The epoch therefore sits in the LAST two words of the record: a torn access
 //    that delivered the words in address order would show stale epoch words, not stale values.
-// Polling is bounded (SyncArea::max_spins).  A wait that expires records the epoch in a host-visible status word and
-// poisons what depended on it with NaN, and the kernel carries on: the grid always drains.  Only fp32-accumulating
-// element types use these kernels (a record has room for two 32-bit values); float64 data takes the streaming kernels.
+// Polling is bounded (SyncArea::max_spins).  When a wait of any lane expires (the workgroup that owes it a record is
+// not resident yet: something else holds part of the device), the whole workgroup leaves the fast path at the next
+// barrier and finishes its tile the slow way (recover_* below): it takes the records that have arrived, RECOMPUTES the
+// others from the kernel's inputs, reads its own rows again from memory and stores its results; a host-visible status
+// word notes that it happened.  Every workgroup publishes its own records before it waits for anybody else's, so
+// workgroups that are scheduled later still find everything they need: the grid always drains and every output is
+// correct, only later.  Only fp32-accumulating element types use these kernels (a record has room for two 32-bit
+// values); float64 data takes the streaming kernels.
 #pragma once
 #include "gn_kernels.h"
 
 namespace gn {
 
 constexpr int kRecFast = 2;  // records a lane keeps in registers while polling
-constexpr int kForcedTimeout = -2;  // poll limit that makes every wait give up at once (tests of the failure path)
+constexpr int kForcedTimeout = -2;  // poll limit that makes every wait give up at once, ready or not, and every record be
+                                    // recomputed (tests of the recovery path)
 constexpr int kTailFast = 2;  // channel records a lane of the dgamma / dbeta stage requests ahead of the dx phase
 constexpr int kMaxResidentBlocksDev = 4 * kNumCU;
+// ADD (forward with fused additions): 0 plain forward; 1 a per-(sample, channel) addend only (same register budget as the plain kernel);
+// 2 a residual tensor, with or without the addend (holds two tiles while it combines them, like the backward).
+constexpr int kAddNone = 0, kAddChannel = 1, kAddResidual = 2;
+// The sum of a forward with fused additions is stored while the rows arrive -- unless it replaces one of its own
+// inputs in place: then it is stored after the exchange, with y, so that a workgroup that has not published its record
+// has not overwritten anything a recomputation of that record would read.
+template <typename T> __device__ __forceinline__ bool sum_after_exchange(const T *x, const AddArgs &add) {
+  return add.sum_out != nullptr && ((const void *)add.sum_out == (const void *)x || (const void *)add.sum_out == add.residual);
+}
 
 struct SyncArea {
-  void *recs;                 // 16-byte records, laid out [N][nchunk][G][tiles]
-  unsigned rec_bytes;
-  void *crecs;                // backward: 16-byte records {S1, S2, epoch} per (sample, tile, channel) of the whole tensor
-  unsigned crec_bytes;
-  void *frecs;                // 16-byte records {value0, value1, epoch} per (sample, group): results of the second level
-  unsigned frec_bytes;        // (two_level != 0 only)
+  void *area;                 // the 16-byte records of the launch, three arrays inside one region of area_bytes bytes:
+  unsigned area_bytes;
+  unsigned rec_first;         // index of the first of the records laid out [N][nchunk][G][tiles]
+  unsigned crec_first;        // backward: records {S1, S2, epoch} per (sample, tile, channel) of the whole tensor
+  unsigned frec_first;        // records {value0, value1, epoch} per (sample, group): results of the second level
   int two_level;              // host side only: selects the TWO_LEVEL instantiation of the kernel
   unsigned long long epoch;   // value that marks "written in this call"
   const unsigned long long *generation;  // device counter that replaces the epoch in captured launches (resident_epoch)
@@ -90,23 +104,25 @@ __device__ __forceinline__ SyncArea resident_epoch(SyncArea s) {
 
 // 128-bit device-scope accesses through a raw buffer descriptor (cache policy sc1)
 constexpr int kAuxDeviceScope = 16;
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t record_buffer(const SyncArea &s) {
-  return __builtin_amdgcn_make_buffer_rsrc(s.recs, 0, (int)s.rec_bytes, 0x27000);
+// One array of records: the buffer descriptor of the whole region (the same for the three arrays, so that it occupies
+// four scalar registers once) and the index of the array's first record in it.
+struct RecordArray {
+  __amdgpu_buffer_rsrc_t rsrc;
+  int first;
+};
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t record_region(const SyncArea &s) {
+  return __builtin_amdgcn_make_buffer_rsrc(s.area, 0, (int)s.area_bytes, 0x27000);
 }
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t channel_record_buffer(const SyncArea &s) {
-  return __builtin_amdgcn_make_buffer_rsrc(s.crecs, 0, (int)s.crec_bytes, 0x27000);
-}
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t final_record_buffer(const SyncArea &s) {
-  return __builtin_amdgcn_make_buffer_rsrc(s.frecs, 0, (int)s.frec_bytes, 0x27000);
-}
-__device__ __forceinline__ void record_store(__amdgpu_buffer_rsrc_t r, int64_t idx, float v0, float v1,
-                                             unsigned long long epoch) {
+__device__ __forceinline__ RecordArray record_buffer(const SyncArea &s) { return {record_region(s), (int)s.rec_first}; }
+__device__ __forceinline__ RecordArray channel_record_buffer(const SyncArea &s) { return {record_region(s), (int)s.crec_first}; }
+__device__ __forceinline__ RecordArray final_record_buffer(const SyncArea &s) { return {record_region(s), (int)s.frec_first}; }
+__device__ __forceinline__ void record_store(const RecordArray &r, int64_t idx, float v0, float v1, unsigned long long epoch) {
   const u32x4 rec = {__builtin_bit_cast(unsigned, v0), __builtin_bit_cast(unsigned, v1), (unsigned)epoch,
                      (unsigned)(epoch >> 32)};
-  __builtin_amdgcn_raw_buffer_store_b128(rec, r, (int)(idx * 16), 0, kAuxDeviceScope);
+  __builtin_amdgcn_raw_buffer_store_b128(rec, r.rsrc, ((int)idx + r.first) * 16, 0, kAuxDeviceScope);
 }
-__device__ __forceinline__ u32x4 record_load(__amdgpu_buffer_rsrc_t r, int64_t idx) {
-  return __builtin_amdgcn_raw_buffer_load_b128(r, (int)(idx * 16), 0, kAuxDeviceScope);
+__device__ __forceinline__ u32x4 record_load(const RecordArray &r, int64_t idx) {
+  return __builtin_amdgcn_raw_buffer_load_b128(r.rsrc, ((int)idx + r.first) * 16, 0, kAuxDeviceScope);
 }
 __device__ __forceinline__ bool record_ready(const u32x4 &rec, unsigned long long epoch) {
   return rec.z == (unsigned)epoch && rec.w == (unsigned)(epoch >> 32);
@@ -130,8 +146,6 @@ __device__ __forceinline__ int record_slot(const PartialGeo &q, int G, int n, in
   return __mul24(__mul24(col, G) + g, q.tiles) + t;
 }
 
-// What a result is replaced by when a wait expired: not a number, so that the call's output cannot pass for one.
-__device__ __forceinline__ float poison() { return __builtin_nanf(""); }
 // Two-level exchange.  With T row tiles per sample every workgroup polls T records for each group of its chunk: fine for a
 // few dozen tiles, but the polling traffic grows with T squared (512 tiles x 16 groups: 8192 records per workgroup, as many
 // bytes as the tensor itself per round of polls).  Beyond a bound set by the host, each group's tile records are instead
@@ -154,21 +168,22 @@ template <typename A> __device__ __forceinline__ void block_sum2(A &a, A &b, A *
   a = (scratch[0] + scratch[1]) + (scratch[2] + scratch[3]);
   b = (scratch[4] + scratch[5]) + (scratch[6] + scratch[7]);
 }
-// Wait for the final record of (sample, group) slot; false (and NaN values) if the wait expires.
-__device__ __forceinline__ void poll_final(const SyncArea &s, __amdgpu_buffer_rsrc_t fb, int slot, float &v0, float &v1) {
+__device__ __forceinline__ void record_values(const u32x4 &rec, float &v0, float &v1) {
+  // copy the lanes out first: __builtin_bit_cast applied directly to a vector element reads element 0
+  const unsigned u0 = rec.x, u1 = rec.y;
+  v0 = __builtin_bit_cast(float, u0);
+  v1 = __builtin_bit_cast(float, u1);
+}
+// Wait for the final record of (sample, group) slot.  If the wait expires, `late` is set and the values mean nothing.
+__device__ __forceinline__ void poll_final(const SyncArea &s, RecordArray fb, int slot, float &v0, float &v1,
+                                           bool &late) {
   int spins = 0;
   while (true) {
     const u32x4 rec = record_load(fb, slot);
-    if (record_ready(rec, s.epoch) && s.max_spins != kForcedTimeout) {
-      const unsigned u0 = rec.x, u1 = rec.y;
-      v0 = __builtin_bit_cast(float, u0);
-      v1 = __builtin_bit_cast(float, u1);
-      return;
-    }
-    if (++spins > s.max_spins) {
-      *s.status = s.epoch;
-      v0 = poison();
-      v1 = poison();
+    record_values(rec, v0, v1);
+    if (record_ready(rec, s.epoch) && s.max_spins != kForcedTimeout) return;
+    if (__builtin_expect(++spins > s.max_spins, 0)) {
+      late = true;
       return;
     }
     __builtin_amdgcn_s_sleep(2);
@@ -176,12 +191,13 @@ __device__ __forceinline__ void poll_final(const SyncArea &s, __amdgpu_buffer_rs
 }
 // Collect the records of group g (all tiles of the chunks that hold a piece of it) with L lanes: each lane polls its
 // own records until they carry this call's epoch, kRecFast at a time (they stay in registers: the round trip that
-// finds them ready also brings their values), and hands (value0, value1, count) of each to body.  If a wait expires,
-// the lane's records are not this call's: body is handed NaN values first, so that whatever the caller accumulates
-// cannot pass for a result.
+// finds them ready also brings their values), and hands (value0, value1, count) of each to body.  If the lane's
+// wait expires, `late` is set and the lane stops: what it has accumulated means nothing, and the workgroup takes the
+// recovery path at its next barrier.
 template <typename BODY>
-__device__ __forceinline__ void for_group_records(const SyncArea &s, __amdgpu_buffer_rsrc_t rb, const PartialGeo &q,
-                                                  const Plan &p, int64_t n, int g, bool valid, int L, int sl, BODY &&body) {
+__device__ __forceinline__ void for_group_records(const SyncArea &s, RecordArray rb, const PartialGeo &q,
+                                                  const Plan &p, int64_t n, int g, bool valid, int L, int sl, bool &late,
+                                                  BODY &&body) {
   int k_lo = 0, nk = 1;
   if (valid) group_chunks(q, p.D, g, k_lo, nk);
   const int P = valid ? q.tiles * nk : 0;
@@ -209,19 +225,446 @@ __device__ __forceinline__ void for_group_records(const SyncArea &s, __amdgpu_bu
       for (int i = 0; i < kRecFast; ++i) ok = ok && (!have[i] || record_ready(rec[i], s.epoch));
       if (s.max_spins == kForcedTimeout) ok = false;
       if (ok) break;
-      if (++spins > s.max_spins) {
-        *s.status = s.epoch;
-        body(poison(), poison(), 1.0f);
-        break;
+      if (__builtin_expect(++spins > s.max_spins, 0)) {
+        late = true;
+        return;
       }
       __builtin_amdgcn_s_sleep(2);
     }
 #pragma unroll
     for (int i = 0; i < kRecFast; ++i) {
       if (have[i]) {
-        // copy the lanes out first: __builtin_bit_cast applied directly to a vector element reads element 0
-        const unsigned u0 = rec[i].x, u1 = rec[i].y;
-        body(__builtin_bit_cast(float, u0), __builtin_bit_cast(float, u1), record_count(p, tt[i], k_lo + kk[i], g));
+        float v0, v1;
+        record_values(rec[i], v0, v1);
+        body(v0, v1, record_count(p, tt[i], k_lo + kk[i], g));
+      }
+    }
+  }
+}
+
+// ---- recovery: a workgroup one of whose waits expired finishes its tile without the fast path -----------------------
+// Cold code, reached by a branch that is uniform over the workgroup, after which the registers of the fast path are
+// dead (the tile is read again from memory).  The workgroup walks the records it needs, 256 at a time: those that
+// have arrived are taken, each of the others is recomputed from the kernel's inputs by all 256 lanes together, with
+// sums in double precision (so that sums of another shape than the fast path's fixed trees lose nothing against
+// them).  A recomputed value is used only if the record has STILL not arrived afterwards: then its workgroup had
+// not published when the recomputation finished reading, hence had not started to write results either (a
+// workgroup does not store results before it has seen its own record through memory, with all the others) -- which
+// matters when the output replaces an input in place.  If the record has arrived meanwhile, the record is taken.
+struct RecoveryLds {
+  float v0[kBlock], v1[kBlock];  // a round of records: values, and whether they had arrived
+  int ok[kBlock];
+  double sums[8];                // cross-wavefront stage of block_sum2_f64
+  int late;                      // set by any lane whose wait expired (the fast path reads it after a barrier)
+  int late_tail;                 // the same for the waits of the dgamma / dbeta stage
+};
+// Rows [r0, r1) of row tile t and channels [c_lo, c_hi) of group g inside chunk k: the elements behind a record.
+struct RecordSpan {
+  int64_t r0, r1;
+  int c_lo, c_hi;
+};
+__device__ __forceinline__ RecordSpan record_span(const Plan &p, int t, int k, int g) {
+  const int cc = p.lpr * p.vec;
+  RecordSpan sp;
+  sp.c_lo = g * p.D > k * cc ? g * p.D : k * cc;
+  sp.c_hi = (g + 1) * p.D < (k + 1) * cc ? (g + 1) * p.D : (k + 1) * cc;
+  if (sp.c_hi > (int)p.C) sp.c_hi = (int)p.C;
+  sp.r0 = (int64_t)t * p.tile_rows;
+  sp.r1 = sp.r0 + p.tile_rows < p.R ? sp.r0 + p.tile_rows : p.R;
+  return sp;
+}
+// Sum of two doubles over the 256 lanes (fixed tree); every lane gets the totals.
+__device__ __forceinline__ void block_sum2_f64(double &a, double &b, double *scratch) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) {
+    const double oa = __shfl_xor(a, m, 64), ob = __shfl_xor(b, m, 64);
+    a += oa;
+    b += ob;
+  }
+  __syncthreads();  // scratch may still be read from a previous use
+  if ((threadIdx.x & 63) == 0) {
+    scratch[threadIdx.x >> 6] = a;
+    scratch[4 + (threadIdx.x >> 6)] = b;
+  }
+  __syncthreads();
+  a = (scratch[0] + scratch[1]) + (scratch[2] + scratch[3]);
+  b = (scratch[4] + scratch[5]) + (scratch[6] + scratch[7]);
+}
+__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+// The kernel's argument block, read again from the kernarg segment through a pointer the compiler cannot see through.
+// A kernel's arguments are loaded where it starts; code at its far end that used those copies would keep them in
+// scalar registers (or spill and restore them) all the way through the fast path.  P must be the kernel's only parameter.
+template <typename P> __device__ __forceinline__ P reread_kernel_args() {
+  static_assert(sizeof(P) % 4 == 0, "whole 32-bit words");
+  const __attribute__((address_space(4))) uint32_t *src =
+      (const __attribute__((address_space(4))) uint32_t *)__builtin_amdgcn_kernarg_segment_ptr();
+  asm volatile("" : "+s"(src));
+  P a;
+  uint32_t *dst = (uint32_t *)&a;
+#pragma unroll
+  for (unsigned i = 0; i < sizeof(P) / 4; ++i) dst[i] = src[i];
+  return a;
+}
+// A zero the compiler cannot see through (see lane_pos).
+__device__ __forceinline__ int opaque_zero() {
+  int z = 0;
+  asm volatile("" : "+s"(z));
+  return z;
+}
+__device__ __forceinline__ float uniform(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
+}
+// One round of the walk: lane i loads record slot_of(e0 + i) (for e0 + i < count) and the round's values and arrival
+// flags are left in LDS for everybody.  arrived(e, rec) decides whether a loaded record counts as there.
+template <typename SLOT, typename ARRIVED>
+__device__ __forceinline__ void load_record_round(RecordArray rb, RecoveryLds &r, int e0, int count, SLOT &&slot_of,
+                                                  ARRIVED &&arrived) {
+  const int e = e0 + (int)threadIdx.x;
+  const bool have = e < count;
+  const u32x4 rec = record_load(rb, have ? slot_of(e) : slot_of(e0));
+  __syncthreads();  // the previous round has been consumed
+  record_values(rec, r.v0[threadIdx.x], r.v1[threadIdx.x]);
+  r.ok[threadIdx.x] = have && arrived(e, rec) ? 1 : 0;
+  __syncthreads();
+}
+// After a recomputation (every lane holds the same v0, v1): look at the record once more and prefer it if it has
+// arrived meanwhile.  Uniform over the workgroup.
+__device__ __forceinline__ void prefer_arrived(const SyncArea &s, RecordArray rb, RecoveryLds &r, int64_t slot,
+                                               float &v0, float &v1) {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // every input the recomputation read is here before the record is read again
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const u32x4 again = record_load(rb, slot);
+    r.ok[0] = record_ready(again, s.epoch) && s.max_spins != kForcedTimeout ? 1 : 0;
+    record_values(again, r.v0[0], r.v1[0]);
+  }
+  __syncthreads();
+  if (uniform(r.ok[0])) {
+    v0 = uniform(r.v0[0]);
+    v1 = uniform(r.v1[0]);
+  }
+  __syncthreads();  // r.*[0] may be rewritten
+}
+
+// Element (row r, channel c) of sample n of the tensor a forward normalises: x, or with fused additions the sum
+// (x + residual) + channel_bias rounded to T once, exactly as the fast path forms it.
+template <typename T, int ADD>
+__device__ __forceinline__ float normalised_input(const T *x, const AddArgs &add, const Plan &p, int64_t n, int64_t r, int c) {
+  using L1 = LaneVec<T, 1>;
+  const int64_t e = (n * p.R + r) * p.C + c;
+  float v[1];
+  L1::unpack(L1::load(x + e), v);
+  if constexpr (ADD != kAddNone) {
+    float vr[1] = {0.f};
+    if (add.residual) L1::unpack(L1::load((const T *)add.residual + e), vr);
+    const float tb = add.channel_bias ? load_scalar<float>(add.channel_bias, n * p.C + c, add.channel_bias_dtype) : 0.f;
+    v[0] = (v[0] + vr[0]) + tb;
+    const typename L1::raw_t packed = L1::pack(v);
+    L1::unpack(packed, v);
+  }
+  return v[0];
+}
+// {mean, M2} of the elements behind forward record (t, k, g) of sample n, by the whole workgroup.
+template <typename T, int ADD>
+__device__ __forceinline__ void recompute_fwd_record(const T *x, const AddArgs &add, const Plan &p, int64_t n, int t, int k,
+                                                     int g, double *scratch, float &mu, float &m2) {
+  const RecordSpan sp = record_span(p, t, k, g);
+  const int nc = sp.c_hi - sp.c_lo;
+  const int64_t cnt = (sp.r1 - sp.r0) * nc;
+  const double K = normalised_input<T, ADD>(x, add, p, n, sp.r0, sp.c_lo);
+  double s1 = 0.0, s2 = 0.0;
+#pragma nounroll
+  for (int64_t i = threadIdx.x; i < cnt; i += kBlock) {
+    const int64_t r = i / nc;
+    const int c = (int)(i - r * nc);
+    const double d = (double)normalised_input<T, ADD>(x, add, p, n, sp.r0 + r, sp.c_lo + c) - K;
+    s1 += d;
+    s2 += d * d;
+  }
+  block_sum2_f64(s1, s2, scratch);
+  const double dm = s1 / (double)cnt;
+  mu = (float)(K + dm);
+  m2 = (float)(s2 - s1 * dm);
+}
+// gamma, and the normalisation coefficients a = rstd gamma, b = beta - mean a, of channel c.
+template <typename PT>
+__device__ __forceinline__ void channel_coeffs(const void *w, const void *b, int c, float mu, float rs, float &gamma, float &a,
+                                               float &bb) {
+  gamma = w ? load_param<PT, float>(w, c) : 1.f;
+  const float beta = b ? load_param<PT, float>(b, c) : 0.f;
+  a = rs * gamma;
+  bb = beta - mu * a;
+}
+// Backward group record (t, k, g) of the sample at xs / dys: {sum_c gamma_c sum g' x, sum_c gamma_c sum g'} with
+// g' = dy act'(x a_c + b_c), by the whole workgroup.  mu, rs: the group's statistics.
+template <typename T, typename PT, int ACT>
+__device__ __forceinline__ void recompute_bwd_record(const T *xs, const T *dys, const void *w, const void *b, const Plan &p,
+                                                     int t, int k, int g, float mu, float rs, double *scratch, float &va,
+                                                     float &vb) {
+  using L1 = LaneVec<T, 1>;
+  const RecordSpan sp = record_span(p, t, k, g);
+  const int nc = sp.c_hi - sp.c_lo;
+  const int64_t cnt = (sp.r1 - sp.r0) * nc;
+  double ta = 0.0, tb = 0.0;
+#pragma nounroll
+  for (int64_t i = threadIdx.x; i < cnt; i += kBlock) {
+    const int64_t r = i / nc;
+    const int c = sp.c_lo + (int)(i - r * nc);
+    float gamma, a, bb, vx[1], vd[1];
+    channel_coeffs<PT>(w, b, c, mu, rs, gamma, a, bb);
+    L1::unpack(L1::load(xs + (sp.r0 + r) * p.C + c), vx);
+    L1::unpack(L1::load(dys + (sp.r0 + r) * p.C + c), vd);
+    const float gp = vd[0] * act_bwd<ACT, float>(vx[0] * a + bb);
+    ta += (double)gamma * ((double)gp * (double)vx[0]);
+    tb += (double)gamma * (double)gp;
+  }
+  block_sum2_f64(ta, tb, scratch);
+  va = (float)ta;
+  vb = (float)tb;
+}
+// Backward channel record (tile t, channel c) of the sample at xs / dys: {sum g' x, sum g'} over the tile's rows.
+template <typename T, int ACT>
+__device__ __forceinline__ void recompute_channel_record(const T *xs, const T *dys, const Plan &p, int t, int c, float a, float bb,
+                                                         double *scratch, float &v0, float &v1) {
+  using L1 = LaneVec<T, 1>;
+  const int64_t r0 = (int64_t)t * p.tile_rows;
+  const int64_t r1 = r0 + p.tile_rows < p.R ? r0 + p.tile_rows : p.R;
+  double S1 = 0.0, S2 = 0.0;
+#pragma nounroll
+  for (int64_t r = r0 + threadIdx.x; r < r1; r += kBlock) {
+    float vx[1], vd[1];
+    L1::unpack(L1::load(xs + r * p.C + c), vx);
+    L1::unpack(L1::load(dys + r * p.C + c), vd);
+    const float gp = vd[0] * act_bwd<ACT, float>(vx[0] * a + bb);
+    S1 += (double)gp * (double)vx[0];
+    S2 += (double)gp;
+  }
+  block_sum2_f64(S1, S2, scratch);
+  v0 = (float)S1;
+  v1 = (float)S2;
+}
+// The records of group g of sample n, one after the other (uniform over the workgroup): body(v0, v1, count) gets each,
+// as it arrived or as recompute(t, k, v0, v1) rebuilt it.
+template <typename BODY, typename RECOMPUTE>
+__device__ __forceinline__ void recover_group_records(const SyncArea &s, RecordArray rb, RecoveryLds &r,
+                                                      const PartialGeo &q, const Plan &p, int64_t n, int g, BODY &&body,
+                                                      RECOMPUTE &&recompute) {
+  int k_lo = 0, nk = 1;
+  group_chunks(q, p.D, g, k_lo, nk);
+  const int P = q.tiles * nk;
+  auto slot_of = [&](int e) {
+    const int kk = e / q.tiles;
+    return record_slot(q, p.G, (int)n, e - kk * q.tiles, k_lo + kk, g);
+  };
+#pragma nounroll
+  for (int e0 = 0; e0 < P; e0 += kBlock) {
+    load_record_round(rb, r, e0, P, slot_of,
+                      [&](int, const u32x4 &rec) { return record_ready(rec, s.epoch) && s.max_spins != kForcedTimeout; });
+    const int m = P - e0 < kBlock ? P - e0 : kBlock;
+#pragma nounroll
+    for (int i = 0; i < m; ++i) {
+      const int e = e0 + i;
+      const int kk = e / q.tiles;
+      const int t = e - kk * q.tiles, k = k_lo + kk;
+      float v0 = uniform(r.v0[i]), v1 = uniform(r.v1[i]);
+      if (!uniform(r.ok[i])) {
+        recompute(t, k, v0, v1);
+        prefer_arrived(s, rb, r, slot_of(e), v0, v1);
+      }
+      body(v0, v1, record_count(p, t, k, g));
+    }
+  }
+}
+
+// The rest of a forward workgroup's work after an expired wait: the statistics of the chunk's groups from the tile
+// records (or from the input where they are missing), then the workgroup's own rows, read again from memory.
+template <typename T, typename PT, int VEC, int ACT, int ADD, bool TWO_LEVEL>
+__device__ __forceinline__ void recover_fwd(const T *x, T *y, const SyncArea &sync, const void *w, const void *b, void *mean_out,
+                                            void *rstd_out, int sdtype, int ydtype, float eps, const AddArgs &add, const Plan &p,
+                                            RecoveryLds &r, float *sm_mu, float *sm_rs) {
+  using LV = LaneVec<T, VEC>;
+  const int salt = opaque_zero();
+  const int64_t n = blockIdx.z + salt;
+  const LanePos l = lane_pos<true>(p, n, false, salt);  // again: nothing of the fast path's is kept alive for this path
+  const PartialGeo q = producer_geo(p);
+  const RecordArray rb = record_buffer(sync);
+  if (threadIdx.x == 0) *sync.status = sync.epoch;
+#pragma nounroll
+  for (int gi = 0; gi < l.ng; ++gi) {
+    const int g = l.g_lo + gi;
+    double nl = 0.0, K = 0.0, s1 = 0.0, s2 = 0.0;
+    recover_group_records(
+        sync, rb, r, q, p, n, g,
+        [&](float mu, float mm, float cnt) {
+          if (nl == 0.0) K = mu;
+          const double d = (double)mu - K;
+          nl += cnt;
+          s1 += cnt * d;
+          s2 += mm + cnt * d * d;
+        },
+        [&](int t, int k, float &v0, float &v1) { recompute_fwd_record<T, ADD>(x, add, p, n, t, k, g, r.sums, v0, v1); });
+    const double dm = s1 / nl;
+    const float gmean = (float)(K + dm);
+    const float rs = (float)(1.0 / sqrt((s2 - s1 * dm) / nl + (double)eps));
+    if (threadIdx.x == 0) {
+      sm_mu[gi] = gmean;
+      sm_rs[gi] = rs;
+      const bool owner = TWO_LEVEL ? owns_group(p, l, gi) : l.tile == 0 && g * p.D >= l.cstart;
+      if (owner) {
+        if (mean_out) store_scalar<float>(mean_out, n * p.G + g, sdtype, gmean);
+        if (rstd_out) store_scalar<float>(rstd_out, n * p.G + g, sdtype, rs);
+        // (two-level exchange: the workgroups that wait for this group's final record get it after all)
+        if (TWO_LEVEL) record_store(final_record_buffer(sync), (int)n * p.G + g, gmean, rs, sync.epoch);
+      }
+    }
+  }
+  __syncthreads();
+  if (l.rows > 0) {
+    float sa[VEC], sb[VEC], unused1[VEC], unused2[VEC], tb[VEC];
+    lane_params_flat<float, PT, VEC>(l.cvi * VEC, w, b, sync.area, sa, sb);
+    lane_coeffs<float, VEC, false>(p, l, sm_mu, sm_rs, nullptr, nullptr, sa, sb, unused1, unused2);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+      tb[j] = ADD != kAddNone && add.channel_bias
+                  ? load_scalar<float>(add.channel_bias, n * p.C + (int64_t)l.cvi * VEC + j, add.channel_bias_dtype)
+                  : 0.f;
+    const int64_t off = (n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC;
+    const int64_t step = (int64_t)p.rpi * p.C;
+    const bool sum_late = sum_after_exchange<T>(x, add);
+#pragma nounroll
+    for (int u = 0; u < l.rows; ++u) {
+      float v[VEC];
+      typename LV::raw_t raw = LV::load(x + off + (int64_t)u * step);
+      LV::unpack(raw, v);
+      if constexpr (ADD != kAddNone) {
+        float vr[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) vr[j] = 0.f;
+        if (add.residual) LV::unpack(LV::load((const T *)add.residual + off + (int64_t)u * step), vr);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] = (v[j] + vr[j]) + tb[j];
+        raw = LV::pack(v);
+        if (add.sum_out && sum_late) store_streaming<LV>((T *)add.sum_out + off + (int64_t)u * step, raw);
+        LV::unpack(raw, v);
+      }
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) v[j] = act_fwd<ACT, float>(v[j] * sa[j] + sb[j]);
+      store_result<T, VEC>(y, off + (int64_t)u * step, v, ydtype);
+    }
+  }
+}
+
+// The same for a backward workgroup, up to and including its rows of dx: the group sums of the chunk's groups from the
+// tile records (or from x and dy where they are missing) give the coefficients, then dx row by row from memory.
+template <typename T, typename PT, int VEC, int ACT, bool TWO_LEVEL>
+__device__ __forceinline__ void recover_bwd_dx(const T *x, const T *dy, T *dx, const void *mean, const void *rstd, int sdtype,
+                                               const void *w, const void *b, const SyncArea &sync, const Plan &p,
+                                               RecoveryLds &r, const float *sm_mu, const float *sm_rs, float *sm_k1,
+                                               float *sm_k2) {
+  using LV = LaneVec<T, VEC>;
+  const int salt = opaque_zero();
+  const int64_t n = blockIdx.z + salt;
+  const LanePos l = lane_pos<true>(p, n, false, salt);  // again: nothing of the fast path's is kept alive for this path
+  const PartialGeo q = producer_geo(p);
+  const RecordArray rb = record_buffer(sync);
+  if (threadIdx.x == 0) *sync.status = sync.epoch;
+  const int64_t sample = n * p.R * p.C;
+#pragma nounroll
+  for (int gi = 0; gi < l.ng; ++gi) {
+    const int g = l.g_lo + gi;
+    const float mu = uniform(sm_mu[gi]), rs = uniform(sm_rs[gi]);
+    double ta = 0.0, tb = 0.0;
+    recover_group_records(
+        sync, rb, r, q, p, n, g,
+        [&](float ra, float rbv, float) {
+          ta += ra;
+          tb += rbv;
+        },
+        [&](int t, int k, float &v0, float &v1) {
+          recompute_bwd_record<T, PT, ACT>(x + sample, dy + sample, w, b, p, t, k, g, mu, rs, r.sums, v0, v1);
+        });
+    const double sc = 1.0 / ((double)p.D * (double)p.R);
+    const double k1 = ((double)mu * tb - ta) * sc * (double)rs * (double)rs * (double)rs;
+    const double k2 = -(double)mu * k1 - tb * sc * (double)rs;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      sm_k1[gi] = (float)k1;
+      sm_k2[gi] = (float)k2;
+      if (TWO_LEVEL && owns_group(p, l, gi)) record_store(final_record_buffer(sync), (int)n * p.G + g, (float)k1, (float)k2, sync.epoch);
+    }
+  }
+  __syncthreads();
+  if (l.rows > 0) {
+    float sa[VEC], sb[VEC], c1[VEC], c2[VEC];
+    lane_params_flat<float, PT, VEC>(l.cvi * VEC, w, b, sync.area, sa, sb);
+    lane_coeffs<float, VEC, true>(p, l, sm_mu, sm_rs, sm_k1, sm_k2, sa, sb, c1, c2);
+    const int64_t off = (n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC;
+    const int64_t step = (int64_t)p.rpi * p.C;
+#pragma nounroll
+    for (int u = 0; u < l.rows; ++u) {
+      float vx[VEC], vd[VEC];
+      LV::unpack(LV::load(x + off + (int64_t)u * step), vx);
+      LV::unpack(LV::load(dy + off + (int64_t)u * step), vd);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) vd[j] = vd[j] * act_bwd<ACT, float>(vx[j] * sa[j] + sb[j]);
+      // (g' passes through T as on the fast path, where it waits in registers in packed form)
+      const typename LV::raw_t gp = LV::pack(vd);
+      LV::unpack(gp, vd);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) vd[j] = sa[j] * vd[j] + (c1[j] * vx[j] + c2[j]);
+      store_streaming<LV>(dx + off + (int64_t)u * step, LV::pack(vd));
+    }
+  }
+}
+
+// dgamma / dbeta of the channels this workgroup finishes, after an expired wait of that stage: every channel record
+// of the whole tensor that feeds them is taken as it arrived, or rebuilt from x and dy.  Records of samples before n0
+// were written by launches that have ended.  x / dy point at sample n0.
+template <typename T, typename PT, int ACT>
+__device__ __forceinline__ void recover_bwd_tail(const T *x, const T *dy, const void *w, const void *b, const void *mean_all,
+                                                 const void *rstd_all, int sdtype, const SyncArea &sync, const Plan &p,
+                                                 RecoveryLds &r, int64_t n0, int64_t n_all, void *dw, void *db) {
+  const int salt = opaque_zero();
+  const LanePos l = lane_pos<true>(p, blockIdx.z + salt, false, salt);
+  const int cpp = kBlock / pow2_ceil_clamped((int)n_all * p.tiles, 64);  // channels per pass of the workgroup, as on the fast path
+  const RecordArray rbc = channel_record_buffer(sync);
+  if (threadIdx.x == 0) *sync.status = sync.epoch;
+  const int pairs = (int)n_all * p.tiles;
+#pragma nounroll
+  for (int cb = l.tile * cpp; cb < l.wch; cb += p.tiles * cpp) {
+#pragma nounroll
+    for (int cc = cb; cc < cb + cpp && cc < l.wch; ++cc) {
+      const int c = l.cstart + cc;
+      const int g = c / p.D;
+      double t1 = 0.0, t2 = 0.0;
+      auto slot_of = [&](int e) { return e * (int)p.C + c; };  // e = sample * tiles + tile
+#pragma nounroll
+      for (int e0 = 0; e0 < pairs; e0 += kBlock) {
+        load_record_round(rbc, r, e0, pairs, slot_of, [&](int e, const u32x4 &rec) {
+          return e / p.tiles < n0 || (record_ready(rec, sync.epoch) && sync.max_spins != kForcedTimeout);
+        });
+        const int m = pairs - e0 < kBlock ? pairs - e0 : kBlock;
+#pragma nounroll
+        for (int i = 0; i < m; ++i) {
+          const int e = e0 + i;
+          const int nn = e / p.tiles, t = e - nn * p.tiles;
+          const float mu = load_scalar<float>(mean_all, (int64_t)nn * p.G + g, sdtype);
+          const float rs = load_scalar<float>(rstd_all, (int64_t)nn * p.G + g, sdtype);
+          float v0 = uniform(r.v0[i]), v1 = uniform(r.v1[i]);
+          if (!uniform(r.ok[i])) {
+            float gamma, a, bb;
+            channel_coeffs<PT>(w, b, c, mu, rs, gamma, a, bb);
+            const int64_t sample = (int64_t)(nn - n0) * p.R * p.C;
+            recompute_channel_record<T, ACT>(x + sample, dy + sample, p, t, c, a, bb, r.sums, v0, v1);
+            prefer_arrived(sync, rbc, r, slot_of(e), v0, v1);
+          }
+          t1 += ((double)v0 - (double)mu * (double)v1) * (double)rs;
+          t2 += (double)v1;
+        }
+      }
+      if (threadIdx.x == 0) {
+        if (dw) store_param<PT, float>(dw, c, (float)t1);
+        if (db) store_param<PT, float>(db, c, (float)t2);
       }
     }
   }
@@ -234,9 +677,6 @@ __device__ __forceinline__ void for_group_records(const SyncArea &s, __amdgpu_bu
 // sums about the lane's own first row.
 //   records : {mean, M2, epoch} per (n, chunk, group, tile)
 // ---------------------------------------------------------------------------------------------
-// ADD: 0 plain forward; 1 a per-(sample, channel) addend only (same register budget as the plain kernel);
-// 2 a residual tensor, with or without the addend (holds two tiles while it combines them, like the backward).
-constexpr int kAddNone = 0, kAddChannel = 1, kAddResidual = 2;
 // Occupancy the register budget is sized for.
 constexpr int fused_fwd_waves(int nv, int add) {
   return add == kAddResidual ? (nv <= 4 ? 4 : nv <= 8 ? 3 : nv <= 16 ? 2 : 1) : (nv <= 8 ? 4 : nv <= 16 ? 3 : 2);
@@ -244,18 +684,37 @@ constexpr int fused_fwd_waves(int nv, int add) {
 // TWO_LEVEL: the exchange of a launch with many row tiles per sample (two_level_exchange on the host).  A template
 // parameter, not a run-time switch: the code of the form a launch does not use would sit in the middle of the path every
 // workgroup executes once, and these kernels are sensitive to their own size.
+// The single parameter of the forward kernel (one block, so that the recovery path can read it again: reread_kernel_args).
+struct FusedFwdParams {
+  const void *x;
+  void *y;
+  SyncArea sync;
+  const void *w, *b;
+  void *mean_out, *rstd_out;
+  int sdtype, ydtype;
+  float eps;
+  int pad_;
+  AddArgs add;
+  Plan p;
+};
 template <typename T, typename PT, int VEC, int ACT, int NV, int ADD, bool TWO_LEVEL>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fwd_waves(NV, ADD)))) void fused_fwd_kernel(
-    const T *__restrict__ x, T *__restrict__ y, SyncArea sync_arg, const void *w, const void *b, void *mean_out,
-    void *rstd_out, int sdtype, int ydtype, acc_t<T> eps, AddArgs add, Plan p) {
+    const FusedFwdParams args) {
   using A = acc_t<T>;
   using LV = LaneVec<T, VEC>;
-  const SyncArea sync = resident_epoch(sync_arg);
+  const T *__restrict__ x = (const T *)args.x;
+  const void *w = args.w, *b = args.b;
+  const AddArgs &add = args.add;
+  const Plan &p = args.p;
+  const SyncArea sync = resident_epoch(args.sync);
   __shared__ A sm0[kBlock * VEC];
   __shared__ A sm1[kBlock * VEC];
+  __shared__ RecoveryLds recovery;
+  if (threadIdx.x == 0) recovery.late = 0;  // (several barriers lie between this and the first lane that may set it)
+  bool late = false;                        // a wait of this lane expired
   const PartialGeo q = producer_geo(p);
   const int64_t n = blockIdx.z;
-  const LanePos l = lane_pos(p, n, false);
+  const LanePos l = lane_pos<true>(p, n, false);
   const int rows = l.rows;
   const int64_t off = (n * p.R + l.row0 + l.ty) * p.C + (int64_t)l.cvi * VEC;
   const int64_t step = (int64_t)p.rpi * p.C;
@@ -267,17 +726,17 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
   A sa[VEC], sb[VEC];
   {
     const int cvi = l.cvi < p.cv ? l.cvi : p.cv - 1;
-    lane_params_flat<A, PT, VEC>(cvi * VEC, w, b, sync.recs, sa, sb);
+    lane_params_flat<A, PT, VEC>(cvi * VEC, w, b, sync.area, sa, sb);
   }
   // ADD: the per-(sample, channel) addend of the lane's channels, requested with the parameters and without branches
   A tb[VEC];
   if constexpr (ADD != kAddNone) {
     const int cvi = l.cvi < p.cv ? l.cvi : p.cv - 1;
-    const void *cb = add.channel_bias ? add.channel_bias : sync.recs;
+    const void *cb = add.channel_bias ? add.channel_bias : sync.area;
     const int64_t cb0 = add.channel_bias ? n * p.C + (int64_t)cvi * VEC : 0;
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
-      const A v = load_scalar_flat<A>(cb, add.channel_bias ? cb0 + j : 0, add.channel_bias_dtype, sync.recs);
+      const A v = load_scalar_flat<A>(cb, add.channel_bias ? cb0 + j : 0, add.channel_bias_dtype, sync.area);
       tb[j] = add.channel_bias ? v : (A)0;
     }
   }
@@ -297,7 +756,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
         buf[u] = LV::load(x + o);
         rbuf[u] = LV::load(rp + o);
       }
-      T *so = (T *)add.sum_out;
+      T *so = sum_after_exchange<T>(x, add) ? nullptr : (T *)add.sum_out;
 #pragma unroll
       for (int u = 0; u < NV; ++u) {
         A vx[VEC], vr[VEC];
@@ -312,7 +771,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
 #pragma unroll
       for (int u = 0; u < NV; ++u) buf[u] = LV::load(x + off + (int64_t)clamp_row(u, rows) * step);
       if constexpr (ADD == kAddChannel) {
-        T *so = (T *)add.sum_out;
+        T *so = sum_after_exchange<T>(x, add) ? nullptr : (T *)add.sum_out;
 #pragma unroll
         for (int u = 0; u < NV; ++u) {
           A vx[VEC];
@@ -365,7 +824,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
       m2[j] = s2[j] - s1[j] * dm;
     }
   }
-  const __amdgpu_buffer_rsrc_t rb = record_buffer(sync);
+  const RecordArray rb = record_buffer(sync);
   trace_point(sync, 1, (float)m2[0]);
   // the reduction and the exchange are one chain of dependent steps that every workgroup of the group waits for:
   // let these wavefronts go first on a SIMD they share with wavefronts of other workgroups that are still streaming
@@ -375,16 +834,29 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
     record_store(rb, record_slot(q, p.G, (int)n, l.tile, l.chunk, g), mu, s2, sync.epoch);
   });
   trace_point(sync, 2);
+  // Each of the two phases that follow works on its own copy of the kernel's arguments, read again where the phase
+  // begins: what the phases before it loaded need not stay in scalar registers (or be spilled and restored) all the way.
+  const unsigned long long epoch = sync.epoch;
+  {
+  const FusedFwdParams args = reread_kernel_args<FusedFwdParams>();
+  const Plan &p = args.p;
+  const PartialGeo q = producer_geo(p);
+  SyncArea sync = args.sync;
+  sync.epoch = epoch;
+  const RecordArray rb = record_buffer(sync);
+  void *mean_out = args.mean_out, *rstd_out = args.rstd_out;
+  const int sdtype = args.sdtype;
+  const A eps = args.eps;
   if constexpr (TWO_LEVEL) {
     // second level: the groups this workgroup owns, one at a time with all 256 lanes (usually one group or none)
-    const __amdgpu_buffer_rsrc_t fb = final_record_buffer(sync);
+    const RecordArray fb = final_record_buffer(sync);
     const A total = (A)p.D * (A)p.R;
     __shared__ A sm_x[12];
     for (int gi = l.tile; gi < l.ng; gi += p.tiles) {  // uniform over the workgroup
       if (!owns_group(p, l, gi)) continue;
       const int g = l.g_lo + gi;
       A nl = (A)0, kl = (A)0, s1 = (A)0, s2 = (A)0;
-      for_group_records(sync, rb, q, p, n, g, true, kBlock, threadIdx.x, [&](float mu, float mm, float cnt) {
+      for_group_records(sync, rb, q, p, n, g, true, kBlock, threadIdx.x, late, [&](float mu, float mm, float cnt) {
         if (nl == (A)0) kl = mu;
         const A d = mu - kl;
         nl += cnt;
@@ -394,6 +866,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
       const A inv = nl > (A)0 ? fast_rcp(nl) : (A)0;
       const A mean_l = kl + s1 * inv;
       const A m2_l = s2 - s1 * s1 * inv;
+      if (late) recovery.late = 1;
       __syncthreads();
       if (threadIdx.x == 0) sm_x[8] = mean_l;  // lane 0 always has a record: the pivot of the merge across lanes
       __syncthreads();
@@ -401,7 +874,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
       const A d = nl > (A)0 ? mean_l - K : (A)0;
       A t1 = nl * d, t2 = m2_l + nl * d * d;
       block_sum2(t1, t2, sm_x);
-      if (threadIdx.x == 0) {
+      if (threadIdx.x == 0 && recovery.late == 0) {  // (after an expired wait the sums mean nothing: the recovery publishes)
         const A dm = t1 * fast_rcp(total);
         const A gmean = K + dm;
         const A rs = fast_rsqrt((t2 - t1 * dm) * fast_rcp(total) + eps);
@@ -413,10 +886,11 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
     // everybody: one final record per group of the chunk
     for (int gi = threadIdx.x; gi < l.ng; gi += kBlock) {
       float gmean, rs;
-      poll_final(sync, fb, (int)n * p.G + l.g_lo + gi, gmean, rs);
+      poll_final(sync, fb, (int)n * p.G + l.g_lo + gi, gmean, rs, late);
       sm0[gi] = gmean;
       sm1[gi] = rs;
     }
+    if (late) recovery.late = 1;
     __syncthreads();
   } else {
     // merge the records of the chunk's groups (exact two-pass form, compute_stats_pt2's job:
@@ -431,7 +905,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
       const int g = l.g_lo + gi;
       // each lane folds its records about the mean of its first one ...
       A nl = (A)0, kl = (A)0, s1 = (A)0, s2 = (A)0;
-      for_group_records(sync, rb, q, p, n, g, valid, L, sl, [&](float mu, float mm, float cnt) {
+      for_group_records(sync, rb, q, p, n, g, valid, L, sl, late, [&](float mu, float mm, float cnt) {
         if (nl == (A)0) kl = mu;
         const A d = mu - kl;
         nl += cnt;
@@ -458,18 +932,40 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
         }
       }
     }
+    if (late) recovery.late = 1;
     __syncthreads();
   }
+  }
   __builtin_amdgcn_s_setprio(0);
+  const FusedFwdParams args2 = reread_kernel_args<FusedFwdParams>();
+  if (__builtin_expect(uniform(recovery.late) != 0, 0)) {
+    // a wait expired somewhere in this workgroup: what the lanes hold means nothing.  Start again from memory.
+    SyncArea ks = args2.sync;
+    ks.epoch = epoch;
+    recover_fwd<T, PT, VEC, ACT, ADD, TWO_LEVEL>((const T *)args2.x, (T *)args2.y, ks, args2.w, args2.b, args2.mean_out,
+                                                 args2.rstd_out, args2.sdtype, args2.ydtype, args2.eps, args2.add, args2.p,
+                                                 recovery, sm0, sm1);
+    return;
+  }
   trace_point(sync, 3);
   if (rows > 0) {
+    const Plan &p = args2.p;
+    const T *x = (const T *)args2.x;
+    T *y = (T *)args2.y;
+    const AddArgs &add = args2.add;
+    const int ydtype = args2.ydtype;
+    const int64_t step = (int64_t)p.rpi * p.C;
     A unused1[VEC], unused2[VEC];
     lane_coeffs<A, VEC, false>(p, l, sm0, sm1, nullptr, nullptr, sa, sb, unused1, unused2);
+    const bool sum_late = ADD != kAddNone && sum_after_exchange<T>(x, add);
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
       if (u < rows) {
         A v[VEC];
         pin(buf[u]);
+        if constexpr (ADD != kAddNone) {
+          if (sum_late) store_streaming<LV>((T *)add.sum_out + off + (int64_t)u * step, buf[u]);
+        }
         LV::unpack(buf[u], v);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) v[j] = act_fwd<ACT, A>(v[j] * sa[j] + sb[j]);
@@ -493,24 +989,48 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
 constexpr int fused_bwd_waves(int nv, int xw) {
   return xw > 0 ? (nv <= 24 ? 3 : 2) : (nv <= 4 ? 4 : nv <= 8 ? 3 : nv <= 22 ? 2 : 1);
 }
+// The single parameter of the backward kernel (see FusedFwdParams).  x, dy, dx, mean, rstd: this launch's samples;
+// mean_all, rstd_all: the whole tensor's; n0: index of this launch's first sample in the tensor, n_all: its samples.
+struct FusedBwdParams {
+  const void *x, *dy;
+  void *dx;
+  const void *mean, *rstd;
+  const void *w, *b;
+  SyncArea sync;
+  void *dw, *db;
+  const void *mean_all, *rstd_all;
+  int64_t n0, n_all;
+  int sdtype, pad_;
+  Plan p;
+};
 template <typename T, typename PT, int VEC, int ACT, int NV, bool TWO_LEVEL, int XW = 0>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bwd_waves(NV, XW)))) void fused_bwd_kernel(
-    const T *__restrict__ x, const T *__restrict__ dy, T *__restrict__ dx, const void *mean, const void *rstd, int sdtype,
-    const void *w, const void *b, SyncArea sync_arg, void *dw, void *db, const void *mean_all, const void *rstd_all,
-    int64_t n0, int64_t n_all, Plan p) {
+    const FusedBwdParams args) {
   using A = acc_t<T>;
   using LV = LaneVec<T, VEC>;
-  const SyncArea sync = resident_epoch(sync_arg);
+  const T *__restrict__ x = (const T *)args.x;
+  const T *__restrict__ dy = (const T *)args.dy;
+  const void *mean = args.mean, *rstd = args.rstd, *w = args.w, *b = args.b;
+  const int64_t n0 = args.n0;
+  const int sdtype = args.sdtype;
+  const Plan &p = args.p;
+  const SyncArea sync = resident_epoch(args.sync);
   __shared__ A sm1[kBlock * VEC];
   __shared__ A sm2[kBlock * VEC];
   __shared__ A sm_mu[kBlock * VEC];
   __shared__ A sm_rs[kBlock * VEC];
+  __shared__ RecoveryLds recovery;
+  if (threadIdx.x == 0) {  // (several barriers lie between this and the first lane that may set either)
+    recovery.late = 0;
+    recovery.late_tail = 0;
+  }
+  bool late = false;  // a wait of this lane expired
   const PartialGeo q = producer_geo(p);
   const int64_t n = blockIdx.z;
-  const LanePos l = lane_pos(p, n, false);
-  const __amdgpu_buffer_rsrc_t rb = record_buffer(sync);
-  const __amdgpu_buffer_rsrc_t rbc = channel_record_buffer(sync);
-  const void *safe = sync.recs;  // readable bytes for loads that only exist to keep the prologue free of branches
+  const LanePos l = lane_pos<true>(p, n, false);
+  const RecordArray rb = record_buffer(sync);
+  const RecordArray rbc = channel_record_buffer(sync);
+  const void *safe = sync.area;  // readable bytes for loads that only exist to keep the prologue free of branches
   const int rows = l.rows;
   const SafeLane sfl = safe_lane<VEC>(p, l, n);
   const int64_t off = sfl.off;
@@ -668,20 +1188,38 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
   }
   __syncthreads();
   trace_point(sync, 2);
+  // The rest of the kernel works on its own copy of the kernel's arguments, read again here: what the phases before it
+  // loaded need not stay in scalar registers (or be spilled and restored) all the way.
+  const unsigned long long epoch = sync.epoch;
+  {
+  const FusedBwdParams args = reread_kernel_args<FusedBwdParams>();
+  const T *x = (const T *)args.x;
+  T *dx = (T *)args.dx;
+  void *dw = args.dw, *db = args.db;
+  const void *mean_all = args.mean_all, *rstd_all = args.rstd_all;
+  const int64_t n0 = args.n0, n_all = args.n_all;
+  const int sdtype = args.sdtype;
+  const Plan &p = args.p;
+  const PartialGeo q = producer_geo(p);
+  SyncArea sync = args.sync;
+  sync.epoch = epoch;
+  const RecordArray rb = record_buffer(sync), rbc = channel_record_buffer(sync);
+  const void *safe = sync.area;
   if constexpr (TWO_LEVEL) {
     // second level (see owns_group): the groups this workgroup owns, one at a time with all 256 lanes
-    const __amdgpu_buffer_rsrc_t fb = final_record_buffer(sync);
+    const RecordArray fb = final_record_buffer(sync);
     __shared__ A sm_x[8];
     for (int gi = l.tile; gi < l.ng; gi += p.tiles) {  // uniform over the workgroup
       if (!owns_group(p, l, gi)) continue;
       const int g = l.g_lo + gi;
       A ta = (A)0, tb = (A)0;
-      for_group_records(sync, rb, q, p, n, g, true, kBlock, threadIdx.x, [&](float ra, float rbv, float) {
+      for_group_records(sync, rb, q, p, n, g, true, kBlock, threadIdx.x, late, [&](float ra, float rbv, float) {
         ta += ra;
         tb += rbv;
       });
+      if (late) recovery.late = 1;
       block_sum2(ta, tb, sm_x);
-      if (threadIdx.x == 0) {
+      if (threadIdx.x == 0 && recovery.late == 0) {  // (after an expired wait the sums mean nothing: the recovery publishes)
         const A mu = sm_mu[gi];
         const A rs = sm_rs[gi];
         const A s = fast_rcp((A)p.D * (A)p.R);
@@ -691,7 +1229,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
     }
     for (int gi = threadIdx.x; gi < l.ng; gi += kBlock) {
       float k1, k2;
-      poll_final(sync, fb, (int)n * p.G + l.g_lo + gi, k1, k2);
+      poll_final(sync, fb, (int)n * p.G + l.g_lo + gi, k1, k2, late);
       sm1[gi] = k1;
       sm2[gi] = k2;
     }
@@ -704,7 +1242,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
       const bool valid = gi < l.ng;
       const int g = l.g_lo + gi;
       A ta = (A)0, tb = (A)0;
-      for_group_records(sync, rb, q, p, n, g, valid, L, sl, [&](float ra, float rbv, float) {
+      for_group_records(sync, rb, q, p, n, g, valid, L, sl, late, [&](float ra, float rbv, float) {
         ta += ra;
         tb += rbv;
       });
@@ -719,6 +1257,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
       }
     }
   }
+  if (late) recovery.late = 1;
   __syncthreads();
   // dgamma / dbeta (compute_dweight_dbias, gn_kernel.cu:695-728).  The workgroups of this launch's first sample
   // share the channels of their chunk: a segment of L lanes per channel sums the channel records of every
@@ -732,6 +1271,19 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
   const int TL = pow2_ceil_clamped(pairs, 64);
   const int tlg = __builtin_ctz(TL);
   const int cpp = kBlock >> tlg;  // channels per pass of the workgroup
+  if (__builtin_expect(uniform(recovery.late) != 0, 0)) {
+    // a wait expired somewhere in this workgroup: what the lanes hold means nothing.  Coefficients, dx and (the
+    // workgroups that finish dgamma / dbeta) the channel sums again, from memory.
+    const FusedBwdParams ka = reread_kernel_args<FusedBwdParams>();
+    SyncArea ks = ka.sync;
+    ks.epoch = epoch;
+    recover_bwd_dx<T, PT, VEC, ACT, TWO_LEVEL>((const T *)ka.x, (const T *)ka.dy, (T *)ka.dx, ka.mean, ka.rstd, ka.sdtype, ka.w, ka.b,
+                                               ks, ka.p, recovery, sm_mu, sm_rs, sm1, sm2);
+    if (blockIdx.z == 0 && (ka.dw || ka.db))
+      recover_bwd_tail<T, PT, ACT>((const T *)ka.x, (const T *)ka.dy, ka.w, ka.b, ka.mean_all, ka.rstd_all, ka.sdtype, ks, ka.p,
+                                   recovery, ka.n0, ka.n_all, ka.dw, ka.db);
+    return;
+  }
   const int tslot = threadIdx.x >> tlg, tsl = threadIdx.x & (TL - 1);
   const bool tail_lane = tail && l.tile * cpp + tslot < l.wch;
   const int tail_c = l.cstart + (tail_lane ? l.tile * cpp + tslot : 0);
@@ -790,6 +1342,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
   trace_point(sync, 4);
   if (tail) {
     int spins = 0;
+    late = false;
     for (int cb = l.tile * cpp; cb < l.wch; cb += p.tiles * cpp) {
       const bool first = cb == l.tile * cpp;
       const int cc = cb + tslot;
@@ -802,17 +1355,15 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
         const int64_t nn = div_by(e, p.by_tiles);
         const int t = e - (int)nn * p.tiles;
         while (valid && nn >= n0 && (!record_ready(rec, sync.epoch) || sync.max_spins == kForcedTimeout)) {
-          if (++spins > sync.max_spins) {
-            *sync.status = sync.epoch;
-            t1 = poison();  // dgamma / dbeta of this channel say so
-            t2 = poison();
+          if (__builtin_expect(++spins > sync.max_spins, 0)) {
+            late = true;  // the sums of this channel mean nothing: the workgroup recomputes its channels below
             break;
           }
           __builtin_amdgcn_s_sleep(2);
           rec = record_load(rbc, (nn * p.tiles + t) * p.C + c);
         }
-        const unsigned u0 = rec.x, u1 = rec.y;
-        const A s1 = __builtin_bit_cast(float, u0), s2 = __builtin_bit_cast(float, u1);
+        A s1, s2;
+        record_values(rec, s1, s2);
         t1 += (s1 - mu * s2) * rs;
         t2 += s2;
       };
@@ -838,6 +1389,16 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
       }
     }
     trace_point(sync, 5);
+    if (late) recovery.late_tail = 1;
+    __syncthreads();
+    if (__builtin_expect(uniform(recovery.late_tail) != 0, 0)) {
+      const FusedBwdParams ka = reread_kernel_args<FusedBwdParams>();
+      SyncArea ks = ka.sync;
+      ks.epoch = epoch;
+      recover_bwd_tail<T, PT, ACT>((const T *)ka.x, (const T *)ka.dy, ka.w, ka.b, ka.mean_all, ka.rstd_all, ka.sdtype, ks, ka.p,
+                                   recovery, ka.n0, ka.n_all, ka.dw, ka.db);
+    }
+  }
   }
 }
 

@@ -5,6 +5,8 @@
 #include <hip/hip_ext.h>
 #include <stddef.h>
 #include <stdint.h>
+#include <tuple>
+#include <utility>
 #include "../../include/gnnhwc.h"
 #include "gn_plan.h"
 
@@ -190,9 +192,23 @@ inline bool one_round_merge(const Plan &p) { return pow2_at_least(p.gmax) <= kBl
 // kernel's begin-to-end time on the device, the quantity a kernel trace reports, with no dispatch gap.
 bool profile_events(int kind, hipEvent_t *start, hipEvent_t *stop);
 
+// GNNHWC_COOPERATIVE=1 (measurement only): the single-launch kernels go through hipLaunchCooperativeKernel, the
+// runtime's own guarantee that a grid is resident as a whole, instead of a plain launch.
+bool cooperative_launches();
+template <typename... KArgs, size_t... I>
+inline void launch_cooperative(void (*kernel)(KArgs...), dim3 grid, dim3 block, hipStream_t stream, std::tuple<KArgs...> &vals,
+                               std::index_sequence<I...>) {
+  void *argv[] = {(void *)&std::get<I>(vals)...};
+  (void)hipLaunchCooperativeKernel((const void *)kernel, grid, block, argv, 0, stream);
+}
 template <typename... KArgs, typename... Args>
 inline void launch(int kind, void (*kernel)(KArgs...), dim3 grid, dim3 block, hipStream_t stream, Args &&...args) {
   hipEvent_t e0 = nullptr, e1 = nullptr;
+  if ((kind == kKindFusedFwd || kind == kKindFusedBwd || kind == kKindFusedFwdAdd) && cooperative_launches()) {
+    std::tuple<KArgs...> vals(static_cast<KArgs>(args)...);
+    launch_cooperative(kernel, grid, block, stream, vals, std::index_sequence_for<KArgs...>{});
+    return;
+  }
   if (profile_events(kind, &e0, &e1))
     hipExtLaunchKernelGGL(kernel, grid, block, 0, stream, e0, e1, 0, static_cast<KArgs>(args)...);
   else

@@ -91,6 +91,7 @@ bool resident_tiling(const Plan &base, int64_t samples, int nv, int slots, Plan 
   const int64_t columns = samples * base.nchunk;
   if (slots <= 0 || columns > slots || samples > 65535) return false;
   if (base.G > 8192 || base.C >= (1 << 23)) return false;  // the kernels index their records with 24-bit multiplies
+  if ((base.lpr & (base.lpr - 1)) != 0) return false;  // ... and find a lane's row and column by shifts
   const int64_t rows = (int64_t)nv * base.rpi;
   const int64_t tiles = (base.R + rows - 1) / rows;
   if (columns * tiles > slots) return false;
@@ -115,13 +116,12 @@ void arm_generation(ResidentWorkspace &r, const CapturedEpoch &c) {
 ResidentWorkspace resident_fwd_ws(void *ws, const Plan &p) {
   ResidentWorkspace r;
   char *base = (char *)ws + kWorkspaceHeader;
-  r.sync.recs = base;
-  r.sync.rec_bytes = (unsigned)resident_rec_bytes(p.G);
-  r.sync.frecs = base + align_up(resident_rec_bytes(p.G), 256);
-  r.sync.frec_bytes = (unsigned)resident_frec_bytes(p.G);
+  r.sync.area = base;
+  r.sync.area_bytes = (unsigned)(resident_fwd_bytes(p.G) - kWorkspaceHeader);
+  r.sync.rec_first = 0;
+  r.sync.frec_first = (unsigned)(align_up(resident_rec_bytes(p.G), 256) / 16);
+  r.sync.crec_first = 0;  // (no channel records in the forward)
   r.sync.two_level = two_level_exchange(p) ? 1 : 0;
-  r.sync.crecs = nullptr;
-  r.sync.crec_bytes = 0;
   r.sync.status = resident_status();
   r.sync.generation = nullptr;
   r.sync.max_spins = resident_spin_limit();
@@ -134,12 +134,11 @@ ResidentWorkspace resident_bwd_ws(void *ws, const Plan &p) {
   ResidentWorkspace r;
   char *base = (char *)ws + kWorkspaceHeader;
   const size_t cc = (size_t)p.lpr * p.vec;
-  r.sync.crecs = base;  // channel records of the whole tensor, [N][tiles][C] x 16 bytes
-  r.sync.crec_bytes = (unsigned)resident_crec_bytes(cc);
-  r.sync.recs = base + resident_crec_bytes(cc);
-  r.sync.rec_bytes = (unsigned)resident_rec_bytes(p.G);
-  r.sync.frecs = base + resident_crec_bytes(cc) + align_up(resident_rec_bytes(p.G), 256);
-  r.sync.frec_bytes = (unsigned)resident_frec_bytes(p.G);
+  r.sync.area = base;
+  r.sync.area_bytes = (unsigned)(resident_bwd_bytes(cc, p.G) - kWorkspaceHeader);
+  r.sync.crec_first = 0;  // channel records of the whole tensor, [N][tiles][C]
+  r.sync.rec_first = (unsigned)(resident_crec_bytes(cc) / 16);
+  r.sync.frec_first = (unsigned)((resident_crec_bytes(cc) + align_up(resident_rec_bytes(p.G), 256)) / 16);
   r.sync.two_level = two_level_exchange(p) ? 1 : 0;
   r.sync.status = resident_status();
   r.sync.generation = nullptr;
@@ -189,11 +188,21 @@ template <typename PT, int ACT, int NV, int ADD> bool try_resident_fwd_nv(const 
     if (add.residual) add.residual = (const elem_t *)add.residual + n0 * sample;
     if (add.sum_out) add.sum_out = (elem_t *)add.sum_out + n0 * sample;
     if (add.channel_bias) add.channel_bias = (const char *)add.channel_bias + n0 * a.plan.C * stat_size(add.channel_bias_dtype);
+    FusedFwdParams k = {};
+    k.x = (const elem_t *)a.x + n0 * sample;
+    k.y = (char *)a.y + n0 * sample * stat_size(a.ydtype);
+    k.sync = r.sync;
+    k.w = a.w;
+    k.b = a.b;
+    k.mean_out = a.mean ? (char *)a.mean + n0 * a.plan.G * stat_size(a.sdtype) : nullptr;
+    k.rstd_out = a.rstd ? (char *)a.rstd + n0 * a.plan.G * stat_size(a.sdtype) : nullptr;
+    k.sdtype = a.sdtype;
+    k.ydtype = a.ydtype;
+    k.eps = (float)a.eps;
+    k.add = add;
+    k.p = pb;
     launch(ADD != kAddNone ? kKindFusedFwdAdd : kKindFusedFwd, r.sync.two_level ? kernel_two : kernel_all, tile_grid(pb, 0),
-           dim3(kBlock), a.stream,
-           (const elem_t *)a.x + n0 * sample, (elem_t *)((char *)a.y + n0 * sample * stat_size(a.ydtype)), r.sync, a.w, a.b,
-           a.mean ? (char *)a.mean + n0 * a.plan.G * stat_size(a.sdtype) : nullptr,
-           a.rstd ? (char *)a.rstd + n0 * a.plan.G * stat_size(a.sdtype) : nullptr, a.sdtype, a.ydtype, (A)a.eps, add, pb);
+           dim3(kBlock), a.stream, k);
   }
   return true;
 }
@@ -271,11 +280,24 @@ template <typename PT, int ACT, int NV, int XW = 0> bool try_resident_bwd_nv(con
     ResidentWorkspace r = resident_bwd_ws(a.ws, pb);
     arm_generation(r, cap);
     const bool last = n0 + per >= a.plan.N;
-    launch(kKindFusedBwd, r.sync.two_level ? kernel_two : kernel_all, tile_grid(pb, 0), dim3(kBlock), a.stream,
-           (const elem_t *)a.x + n0 * sample,
-           (const elem_t *)a.dy + n0 * sample, (elem_t *)a.dx + n0 * sample, (const char *)a.mean + n0 * a.plan.G * ssz,
-           (const char *)a.rstd + n0 * a.plan.G * ssz, a.sdtype, a.w, a.b, r.sync, last ? a.dw : nullptr,
-           last ? a.db : nullptr, a.mean, a.rstd, n0, a.plan.N, pb);
+    FusedBwdParams k = {};
+    k.x = (const elem_t *)a.x + n0 * sample;
+    k.dy = (const elem_t *)a.dy + n0 * sample;
+    k.dx = (elem_t *)a.dx + n0 * sample;
+    k.mean = (const char *)a.mean + n0 * a.plan.G * ssz;
+    k.rstd = (const char *)a.rstd + n0 * a.plan.G * ssz;
+    k.w = a.w;
+    k.b = a.b;
+    k.sync = r.sync;
+    k.dw = last ? a.dw : nullptr;
+    k.db = last ? a.db : nullptr;
+    k.mean_all = a.mean;
+    k.rstd_all = a.rstd;
+    k.n0 = n0;
+    k.n_all = a.plan.N;
+    k.sdtype = a.sdtype;
+    k.p = pb;
+    launch(kKindFusedBwd, r.sync.two_level ? kernel_two : kernel_all, tile_grid(pb, 0), dim3(kBlock), a.stream, k);
   }
   return true;
 }

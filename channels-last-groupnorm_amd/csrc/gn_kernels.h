@@ -35,25 +35,31 @@ struct LanePos {
 };
 // `reversed` walks the row tiles from the far end in blocks of eight: the second pass of a two-pass
 // operation then starts on the tiles the first pass touched last, while tile t stays on XCD t mod 8.
-__device__ __forceinline__ LanePos lane_pos(const Plan &p, int64_t n, bool reversed) {
+// `salt` is zero.  A caller that needs the position a second time, late in a kernel, passes a zero the compiler
+// cannot see through, so that the position is computed again there instead of being kept in registers all the way.
+// POW2: the chunk width p.lpr (and with it p.rpi) is known to be a power of two: shifts instead of divisions, and the two
+// divisors need not be loaded.
+template <bool POW2 = false>
+__device__ __forceinline__ LanePos lane_pos(const Plan &p, int64_t n, bool reversed, int salt = 0) {
   LanePos l;
   l.n = n;
-  int t = blockIdx.x;
+  int t = blockIdx.x + salt;
   if (reversed) {
     const int full = p.tiles & ~7;
     if (t < full) t = full - 8 - (t & ~7) + (t & 7);
   }
   l.tile = t;
-  l.chunk = blockIdx.y;
-  const int tid = threadIdx.x;
-  l.ty = div_by(tid, p.by_lpr);
-  l.tx = tid - l.ty * p.lpr;
+  l.chunk = blockIdx.y + salt;
+  const int tid = threadIdx.x + salt;
+  const int lpr_log2 = __builtin_ctz(p.lpr);
+  l.ty = POW2 ? tid >> lpr_log2 : div_by(tid, p.by_lpr);
+  l.tx = POW2 ? tid & (p.lpr - 1) : tid - l.ty * p.lpr;
   l.cvi = l.chunk * p.lpr + l.tx;
   l.row0 = (int64_t)l.tile * p.tile_rows;
   const int64_t rem = p.R - l.row0;
   l.len = rem < p.tile_rows ? (int)rem : p.tile_rows;
-  l.rows_base = div_by(l.len, p.by_rpi);
-  l.rows_rem = l.len - l.rows_base * p.rpi;
+  l.rows_base = POW2 ? l.len >> __builtin_ctz(p.rpi) : div_by(l.len, p.by_rpi);
+  l.rows_rem = POW2 ? l.len & (p.rpi - 1) : l.len - l.rows_base * p.rpi;
   l.cstart = l.chunk * p.lpr * p.vec;
   const int lanes_here = p.cv - l.chunk * p.lpr < p.lpr ? p.cv - l.chunk * p.lpr : p.lpr;
   l.wch = lanes_here * p.vec;

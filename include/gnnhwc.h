@@ -22,7 +22,7 @@
  * State the library keeps (none of it affects results): a per-thread error string; and, for the single-launch
  * kernels (see gnnhwc_set_resident), process-wide: the on / off switch, per device the stream of the last
  * single-launch call and one event that orders a call on another stream behind it, a 64-byte host-pinned status
- * word (allocated with hipHostMalloc at the first single-launch call of the process), one 8-byte generation cell per
+ * word (allocated with hipHostMalloc at the first single-launch call of the process; see gnnhwc_resident_status), one 8-byte generation cell per
  * device inside the library's image (used by launches recorded into HIP graphs), a pool of events while
  * gnnhwc_profile_enable is on, and a device buffer of 64 KiB when GNNHWC_TRACE is set in the environment.
  * A caller that must see no allocation at all after start-up either makes one warm-up call per device first or
@@ -209,12 +209,13 @@ int gnnhwc_bwd_nchw(const void *dy, const void *x, const void *weight, const voi
  * Kernel selection (no counterpart in the reference).  By default a problem whose tensors fit in the
  * register files of one launch is run by the single-launch kernels (x and dy are read from memory once;
  * workgroups exchange partial results while resident), anything else by the multi-launch streaming
- * kernels.  A single-launch kernel needs the device to itself among its kind: calls of one process on
+ * kernels.  A single-launch kernel is fastest with the device to itself: calls of one process on
  * different streams are ordered by the library (a call on another stream than the previous single-launch
  * call of the device first makes its stream wait, on the device, for what has been submitted to that
- * previous stream), but launches recorded into graphs that are replayed concurrently, and other processes
- * on the same device, are not; gnnhwc_set_resident(0) (or GNNHWC_DISABLE_RESIDENT=1 in the environment)
- * forces the streaming kernels, which have no such requirement.  Process-wide; returns the previous setting.
+ * previous stream).  Where the device is shared all the same (launches recorded into graphs that are replayed
+ * concurrently, other processes), the kernels still produce correct results, more slowly (see
+ * gnnhwc_resident_status below); gnnhwc_set_resident(0) (or GNNHWC_DISABLE_RESIDENT=1 in the environment)
+ * selects the streaming kernels, which do not care.  Process-wide; returns the previous setting.
  */
 int gnnhwc_set_resident(int on);
 
@@ -237,21 +238,26 @@ int gnnhwc_profile_collect(int64_t *launches /* [GNNHWC_NUM_KERNEL_KINDS] */,
 const char *gnnhwc_kernel_kind_name(int kind);
 
 /*
- * Failure handling of the single-launch kernels (no counterpart in the reference).  Their workgroups wait for
- * each other with a bounded number of polls.  If a wait expires (the workgroups were not all resident at once: another
- * process or a concurrently replayed graph held part of the device), the kernel still ends normally, and
- *   - everything that depended on the expired wait is written as NaN: mean / rstd of the group, every y (dx) element
- *     of the tiles that waited for it, dweight / dbias of the channels concerned.  The output of the failed call
- *     cannot be mistaken for a result;
- *   - a host-visible status word is set.  gnnhwc_resident_status() reads and clears it: it returns GNNHWC_OK, or
- *     GNNHWC_ERR_LAUNCH (with a message) if a single-launch kernel of this process has failed since the last check.
- *     It does not synchronise: call it once the work in question has completed (after a stream or event
- *     synchronisation, after a graph replay has finished).  The next gnnhwc_fwd / gnnhwc_bwd / gnnhwc_fwd_nchw /
- *     gnnhwc_bwd_nchw call on any thread performs the same check, returns that error without launching anything,
- *     and the process uses the multi-launch kernels from then on.
- * gnnhwc_debug_set_spin_limit sets the number of polls per wait and returns the previous value: negative restores the
- * default (2^20, about a second), except -2, which makes every wait give up at its first poll whether or not the
- * data had arrived; tests use that to exercise this path, every kernel still exits normally.
+ * What the single-launch kernels do when their workgroups cannot all run at once (no counterpart in the reference,
+ * whose independent launches, gn_kernel.cu:439-536 and 932-1060, have no such state -- and neither has this library: no
+ * call fails or returns wrong numbers because of it).  The workgroups of such a kernel wait for each other's partial
+ * results with a bounded number of polls.  If a wait expires (another stream, a concurrently replayed graph or another
+ * process holds part of the device, so that some workgroups have not been scheduled yet), the waiting workgroup stops
+ * waiting: it takes the partial results that have arrived, recomputes the missing ones from the call's own inputs,
+ * reads its rows again and stores its results.  Every workgroup publishes its own partial results before it waits, so
+ * the workgroups scheduled later find everything: the kernel always ends, and y, mean, rstd, dx, dweight, dbias are
+ * correct to the same tolerances as always -- the call only takes longer (milliseconds instead of microseconds when
+ * many workgroups had to recompute).
+ *   - gnnhwc_resident_status() returns 1 if that has happened in any single-launch kernel of this process since the
+ *     last query, else 0, and clears the note.  It never reports an error and does not synchronise: ask once the work
+ *     in question has completed.  A caller that sees 1 often may prefer gnnhwc_set_resident(0) for that workload
+ *     (the multi-launch kernels need no co-residency); nothing switches by itself.
+ *   - gnnhwc_debug_set_spin_limit sets the number of polls per wait (about a microsecond each) and returns the
+ *     previous value: negative restores the default (1024), except -2, which makes every wait expire at its first poll
+ *     whether or not the data had arrived and every partial result be recomputed; tests use that to exercise the
+ *     recovery, every kernel still exits normally.  With -2, outputs must not replace inputs in place (a recomputation
+ *     that ignores what has arrived may read rows another workgroup has already overwritten; in normal operation a
+ *     recomputed value is only used if its workgroup has provably not written anything yet).
  */
 int gnnhwc_resident_status(void);
 int gnnhwc_debug_set_spin_limit(int polls);
