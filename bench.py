@@ -17,6 +17,7 @@ torch.cuda.synchronize() calls.  Prints ONE JSON line:
   copy_ceiling the library's plain copy kernel on tensors of each shape's size: what a kernel with no
                arithmetic and no cross-workgroup dependency reaches at that size on this GPU
   cpu_baseline torch.nn.functional.group_norm + SiLU + autograd on the host cores, same tensors (bounded sample)
+  torch_gpu    the same torch expression on the same GPU and the same channels-last tensors, us per call (context only)
   shapes       per-shape us/call and GB/s, with warm (same buffers every call) and cold (rotating through
                > 512 MB of distinct buffers) figures
 """
@@ -46,6 +47,7 @@ def parse_args():
     ap.add_argument("--workload", default="sd_unet")
     ap.add_argument("--all", action="store_true", help="also time every other configuration (reported under 'shapes')")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-torch-gpu", action="store_true", help="skip the torch-on-the-same-GPU context leg")
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-shape warm / cold / copy-ceiling table")
     ap.add_argument("--graph", action="store_true", help="time the replay of a HIP graph of the K steps instead of eager launches")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
@@ -483,6 +485,35 @@ def switch_cost(names, device):
               ("after a 1 MB GroupNorm forward", lambda: small.step(0, stream, "fwd")))
     print("# event-timed microseconds per launch; same buffers every launch")
     print("%-6s %-4s %-12s %14s %26s %32s" % ("shape", "pass", "kernel", others[0][0], others[1][0], others[2][0]))
+    # the plain copy kernel (a few hundred bytes of code) on 10 MB, as the kernel that is timed: what a switch costs a
+    # kernel whose code is negligible (its "different kernel" is the small GroupNorm forward in both columns)
+    big_src = torch.empty((10 << 20,), dtype=torch.uint8, device=device)
+    big_dst = torch.empty_like(big_src)
+
+    def big_copy():
+        _cabi.check(_cabi.lib.gnnhwc_debug_copy(big_dst.data_ptr(), big_src.data_ptr(), big_src.numel(), stream), "gnnhwc_debug_copy")
+
+    row = []
+    for other in (None, lambda: small.step(0, stream, "fwd"), lambda: small.step(0, stream, "fwd")):
+        def it(profile):
+            if other is not None:
+                other()
+            _cabi.profile_enable(profile)
+            big_copy()
+            _cabi.profile_enable(False)
+        for _ in range(50):
+            it(False)
+        torch.cuda.synchronize()
+        _cabi.profile_collect()
+        best = None
+        for _ in range(3):
+            for _ in range(100):
+                it(True)
+            torch.cuda.synchronize()
+            res = {k: ms / n * 1e3 for k, (n, ms) in _cabi.profile_collect().items() if n}
+            best = res["copy"] if best is None else min(best, res["copy"])
+        row.append(best)
+    print("%-6s %-4s %-12s %14.2f %26.2f %32.2f" % ("10MB", "-", "copy", row[0], row[1], row[2]))
     for name in names:
         p = Problem(configs.CONFIGS[name], device)
         for which in (("fwd", "bwd") if p.bwd else ("fwd",)):
@@ -794,6 +825,43 @@ def nchw_table(names, device, steps, warmup):
     return out
 
 
+def torch_gpu_leg(names, device, steps, warmup):
+    """Context only, never a target: torch's own GroupNorm followed by the activation (and their autograd backward) on
+    the same GPU and the same channels-last tensors -- the comparison the reference's benchmark makes
+    (benchmark.py:48-49, 86-96).  us per call, forward and forward + backward."""
+    import torch
+    import torch.nn.functional as F
+    import workloads as configs
+
+    acts = {"identity": lambda t: t, "relu": F.relu, "silu": F.silu, "gelu": F.gelu,
+            "gelu_tanh": lambda t: F.gelu(t, approximate="tanh")}
+    out = {}
+    for n in names:
+        cfg = configs.CONFIGS[n]
+        inp = configs.make_inputs(cfg, device)
+        xt = inp["x"].detach().clone(memory_format=torch.preserve_format).requires_grad_()  # (N, C, *spatial), channels fastest
+        wt, bt = inp["w"].clone().requires_grad_(), inp["b"].clone().requires_grad_()
+        dyt = inp["dy"]
+        act = acts[cfg.act]
+
+        def fwd():
+            with torch.no_grad():
+                act(F.group_norm(xt, cfg.G, wt, bt, 1e-5))
+
+        def fwd_bwd():
+            yt = act(F.group_norm(xt, cfg.G, wt, bt, 1e-5))
+            torch.autograd.grad(yt, (xt, wt, bt), dyt)
+
+        r = {"fwd_us": round(min(time_region(fwd, steps, warmup, False) for _ in range(3)) / steps * 1e6, 2)}
+        if cfg.passes != "fwd":
+            r["fwd_bwd_us"] = round(min(time_region(fwd_bwd, steps, warmup, False) for _ in range(3)) / steps * 1e6, 2)
+        out[n] = r
+        del xt, dyt
+        torch.cuda.empty_cache()
+    return {"what": "torch.nn.functional.group_norm + activation (+ autograd.grad) on the same GPU, same channels-last "
+                    "tensors, eager; context only", "us_per_call": out}
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -952,6 +1020,8 @@ def main():
         line["cast"] = cast_table(head_names, device, max(20, args.steps // 2), args.warmup)
     if args.fused_add:
         line["fused_add"] = fused_add_table(head_names, device, max(20, args.steps // 2), args.warmup)
+    if not args.no_torch_gpu:
+        line["torch_gpu"] = torch_gpu_leg(head_names, device, max(10, args.steps // 4), min(args.warmup, 5))
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(head_names, args.cpu_seconds)
     print(json.dumps(line))

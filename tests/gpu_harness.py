@@ -88,6 +88,33 @@ def err(a, truth):
     return float(((a - t).abs() / (t.abs() + rms)).max())
 
 
+def rel_err(a, truth):
+    """max_i |a_i - t_i| / |t_i| over the elements of typical size, |t_i| >= rms(t): the pure relative error, where
+    it is meaningful (near zero a ratio says nothing about accuracy; err() above covers those elements)."""
+    a = torch.as_tensor(a).detach().to("cpu", torch.float64).reshape(-1)
+    t = torch.as_tensor(truth).detach().to("cpu", torch.float64).reshape(-1)
+    assert a.shape == t.shape, (a.shape, t.shape)
+    if t.numel() == 0:
+        return 0.0
+    rms = float(t.square().mean().sqrt())
+    big = t.abs() >= rms
+    if rms == 0.0 or not bool(big.any()):
+        return 0.0
+    return float(((a - t).abs()[big] / t.abs()[big]).max())
+
+
+# Observed errors, one JSON object per line, for the per-configuration result table (profiles/results_all_configs.txt is
+# built from it).  Written only when GNNHWC_PARITY_LOG names a file.
+def record_errors(**fields):
+    import json
+    import os
+
+    path = os.environ.get("GNNHWC_PARITY_LOG")
+    if path:
+        with open(path, "a") as f:
+            f.write(json.dumps(fields) + "\n")
+
+
 def as_np64(t):
     return t.detach().to("cpu", torch.float64).numpy()
 

@@ -2,7 +2,8 @@
 and against torch's own GroupNorm + activation on the same seeded inputs.
 
 Tolerances (the build's stated bar):
-  fp32 / fp64 : err <= 1e-5 (fp64: 1e-12), with err = max |ours - truth| / (|truth| + rms(truth));
+  fp32 / fp64 : err <= 1e-5 (fp64: 1e-12), with err = max |ours - truth| / (|truth| + rms(truth)), AND the pure relative
+                error max |ours - truth| / |truth| over the elements with |truth| >= rms(truth) within the same bound;
   fp16 / bf16 : err(ours vs float64 truth) <= err(torch's own fp16/bf16 GroupNorm+activation vs the same truth)
                 times (1 + HALF_SLACK) -- i.e. no worse than the library routine's own half-precision error.
 relu's derivative is discontinuous at 0: dx elements whose pre-activation is within RELU_BAND of 0 are
@@ -15,7 +16,7 @@ import torch
 from oracle import gn_oracle as orc
 from tests import configs
 from gnnhwc import _cabi
-from tests.gpu_harness import as_np64, cabi_bwd, cabi_fwd, err, nrc_view
+from tests.gpu_harness import as_np64, cabi_bwd, cabi_fwd, err, nrc_view, record_errors, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -48,19 +49,29 @@ def _relu_mask(inp, truth, G):
     return np.abs(z) > RELU_BAND
 
 
-def _check(name, ours, truth, lib_result, dtype, mask=None):
+def _check(name, ours, truth, lib_result, dtype, mask=None, log=None):
+    """Asserts the bars and returns the observed err.  log: a dict the observed figures are added to, under `name`."""
     o, t = as_np64(ours) if isinstance(ours, torch.Tensor) else ours, truth
     if mask is not None:
         o, t = np.where(mask, o, 0.0), np.where(mask, t, 0.0)
     e = err(o, t)
+    r = rel_err(o, t)
+    bar = None
     if dtype == torch.float32:
+        bar = FP32_TOL
         assert e <= FP32_TOL, "%s: err %.3g > %.1g" % (name, e, FP32_TOL)
+        assert r <= FP32_TOL, "%s: relative error %.3g > %.1g" % (name, r, FP32_TOL)
     elif dtype == torch.float64:
+        bar = FP64_TOL
         assert e <= FP64_TOL, "%s: err %.3g > %.1g" % (name, e, FP64_TOL)
+        assert r <= FP64_TOL, "%s: relative error %.3g > %.1g" % (name, r, FP64_TOL)
     else:
         l = lib_result if mask is None else np.where(mask, lib_result, 0.0)
         e_lib = err(l, t)
-        assert e <= e_lib * (1 + HALF_SLACK), "%s: err %.3g vs torch's own %s error %.3g" % (name, e, dtype, e_lib)
+        bar = e_lib * (1 + HALF_SLACK)
+        assert e <= bar, "%s: err %.3g vs torch's own %s error %.3g" % (name, e, dtype, e_lib)
+    if log is not None:
+        log[name] = {"err": e, "rel": r, "bar": bar}
     return e
 
 
@@ -76,17 +87,20 @@ def test_config_parity(family, name, device):
     lib = _torch_same_dtype(inp, cfg.G, cfg.act) if dtype in (torch.float16, torch.bfloat16) else None
     y, mean, rstd = cabi_fwd(x, inp["w"], inp["b"], cfg.G, EPS, act)
     torch.cuda.synchronize()
-    _check("mean", mean, truth["mean"], None, torch.float32 if dtype != torch.float64 else dtype)
-    _check("rstd", rstd, truth["rstd"], None, torch.float32 if dtype != torch.float64 else dtype)
-    _check("y", y, truth["y"], lib and lib["y"], dtype)
+    log = {}
+    _check("mean", mean, truth["mean"], None, torch.float32 if dtype != torch.float64 else dtype, log=log)
+    _check("rstd", rstd, truth["rstd"], None, torch.float32 if dtype != torch.float64 else dtype, log=log)
+    _check("y", y, truth["y"], lib and lib["y"], dtype, log=log)
     if cfg.passes == "fwd":
+        record_errors(config=name, family=family, dtype=cfg.dtype, observed=log)
         return
     dx, dw, db = cabi_bwd(dy, x, inp["w"], inp["b"], mean, rstd, cfg.G, act)
     torch.cuda.synchronize()
     mask = _relu_mask(inp, truth, cfg.G) if cfg.act == "relu" else None
-    _check("dx", dx, truth["dx"], lib and lib["dx"], dtype, mask)
-    _check("dw", dw, truth["dw"], lib and lib["dw"], dtype)
-    _check("db", db, truth["db"], lib and lib["db"], dtype)
+    _check("dx", dx, truth["dx"], lib and lib["dx"], dtype, mask, log=log)
+    _check("dw", dw, truth["dw"], lib and lib["dw"], dtype, log=log)
+    _check("db", db, truth["db"], lib and lib["db"], dtype, log=log)
+    record_errors(config=name, family=family, dtype=cfg.dtype, observed=log)
     # size-independent property: dx sums to zero over every (n, g) slab, relative to the slab's absolute sum
     N, R, C = x.shape
     slab = as_np64(dx).reshape(N, R, cfg.G, C // cfg.G)
