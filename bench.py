@@ -12,7 +12,7 @@ torch.cuda.synchronize() calls.  Prints ONE JSON line:
   roofline     the dominant kernel (the kernel kind and shape the step spends the largest share of its kernel time
                in: mean launch duration x launches per step): its algorithmic bytes / its mean duration, measured
                here with HIP events bound to every launch on the launch stream, against 8 TB/s; every kernel's share
-               and fraction is listed under `kernels`; `traffic` is read from profiles/hbm_traffic_sd_unet.txt
+               and fraction is listed under `kernels`; `traffic` is read from profiles/results_all_configs.txt
                (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --counter-workload`), null when absent
   copy_ceiling the library's plain copy kernel on tensors of each shape's size: what a kernel with no
                arithmetic and no cross-workgroup dependency reaches at that size on this GPU
@@ -73,6 +73,13 @@ def parse_args():
                          "first load 0, 1, 2, 3 copies of the library under other names, which moves the code of the library proper "
                          "by one 2 MB slot each: how much of a kernel's time depends on where the loader put its code")
     ap.add_argument("--code-placement-child", type=int, default=-1, help=argparse.SUPPRESS)
+    ap.add_argument("--results-table", action="store_true",
+                    help="no headline: print the per-configuration result table (timings measured now; counter traffic and parity "
+                         "errors read from the files named by --pmc-plan, --pmc-fetch, --pmc-write and --parity-log)")
+    ap.add_argument("--pmc-plan", help="stdout of a `--counter-workload` run (its JSON line says which dispatches belong to which configuration)")
+    ap.add_argument("--pmc-fetch", help="counter_collection CSV of the rocprofv3 --pmc FETCH_SIZE run")
+    ap.add_argument("--pmc-write", help="counter_collection CSV of the rocprofv3 --pmc WRITE_SIZE run")
+    ap.add_argument("--parity-log", help="JSON lines written by tests/test_gpu_parity.py with GNNHWC_PARITY_LOG set")
     ap.add_argument("--counter-workload", action="store_true",
                     help="no timing: one 256 MiB plain copy (calibration) and a few fwd+bwd calls per shape, for a rocprofv3 --pmc run")
     return ap.parse_args()
@@ -137,6 +144,16 @@ class Problem:
                                  self.ws_b.data_ptr(), self.ws_b.numel(), stream)
         if rc != 0:
             raise RuntimeError(self.lib.gnnhwc_last_error().decode())
+
+    def instance(self, which):
+        """Name of the kernel instance the library launches for this problem's forward / backward, from a call made now:
+        e.g. fused_bwd,rows=22,window=0,two_level=0,launches=1 or multi-launch."""
+        import torch
+        from gnnhwc import _cabi
+
+        stream = torch.cuda.current_stream().cuda_stream
+        (self.fwd if which == "fwd" else self.bwd_)(0, stream)
+        return _cabi.last_launch().replace(" ", ",")
 
     def step(self, s, stream, which="both"):
         if which in ("both", "fwd"):
@@ -267,22 +284,36 @@ def copy_ceiling(nbytes, device, steps):
     return 2 * n / (t / steps) / 1e9
 
 
-TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_sd_unet.txt")
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "results_all_configs.txt")
 
 
 def recorded_traffic():
-    """{(shape, kind): (fetch_bytes, write_bytes)} from the lines `TRAFFIC <shape> <kind> <fetch> <write>` of the
-    committed counter summary, or {} when there is none."""
+    """{(shape, kind): (fetch_bytes, write_bytes, instance)} from the lines `TRAFFIC <shape> <kind> <fetch> <write>
+    <instance>` of the committed counter summary, or {} when there is none.  `instance` names the kernel the counters
+    were taken on (rows per lane, window, exchange form: Problem.instance()); a figure whose instance is not the one
+    this build launches for the shape is stale and is not reported."""
     out = {}
     try:
         with open(TRAFFIC_FILE) as f:
             for ln in f:
                 w = ln.split()
-                if len(w) == 5 and w[0] == "TRAFFIC":
-                    out[(w[1], w[2])] = (float(w[3]), float(w[4]))
+                if len(w) >= 5 and w[0] == "TRAFFIC":
+                    out[(w[1], w[2])] = (float(w[3]), float(w[4]), w[5] if len(w) > 5 else "")
     except OSError:
         pass
     return out
+
+
+def traffic_of(traffic, prob, kind):
+    """Recorded traffic (bytes per launch) of `kind` on prob's shape if it was taken on the kernel instance this build
+    launches, else None and why."""
+    rec = traffic.get((prob.cfg.name, kind))
+    if rec is None:
+        return None, "not recorded"
+    now = prob.instance("bwd" if "bwd" in kind else "fwd")
+    if rec[2] != now:
+        return None, "stale: recorded on %s, this build launches %s" % (rec[2] or "an unnamed instance", now)
+    return rec[0] + rec[1], None
 
 
 def counter_workload(probs, device):
@@ -298,11 +329,33 @@ def counter_workload(probs, device):
     for _ in range(3):
         _cabi.check(_cabi.lib.gnnhwc_debug_copy(dst.data_ptr(), src.data_ptr(), n, stream), "gnnhwc_debug_copy")
     torch.cuda.synchronize()
+    plan = []
+    mark_src = torch.zeros((16,), dtype=torch.uint8, device=device)
+    mark_dst = torch.zeros_like(mark_src)
     for p in probs:
+        # a 16-byte plain copy (one workgroup) in front of every configuration: the marker that cuts the dispatch sequence
+        _cabi.check(_cabi.lib.gnnhwc_debug_copy(mark_dst.data_ptr(), mark_src.data_ptr(), 16, stream), "gnnhwc_debug_copy")
+        # one call first, with the library's own launch count: how many dispatches a forward and a backward of this shape are
+        _cabi.profile_collect()
+        _cabi.profile_enable(True)
+        p.step(0, stream, "fwd")
+        _cabi.profile_enable(False)
+        nf = sum(v[0] for v in _cabi.profile_collect().values())
+        fi = _cabi.last_launch().replace(" ", ",")
+        nb, bi = 0, None
+        if p.bwd:
+            _cabi.profile_enable(True)
+            p.step(0, stream, "bwd")
+            _cabi.profile_enable(False)
+            nb = sum(v[0] for v in _cabi.profile_collect().values())
+            bi = _cabi.last_launch().replace(" ", ",")
         for _ in range(5):
             p.step(0, stream)
         torch.cuda.synchronize()
-    print(json.dumps({"counter_workload": [p.cfg.name for p in probs], "copy_bytes": n}))
+        plan.append({"name": p.cfg.name, "S": p.S, "fwd_dispatches": nf, "bwd_dispatches": nb, "fwd_instance": fi, "bwd_instance": bi})
+    # dispatch order: 3 plain copies of copy_bytes, then per configuration a one-workgroup marker copy and several calls, each
+    # `fwd_dispatches` forward launches followed by `bwd_dispatches` backward launches
+    print(json.dumps({"counter_workload": plan, "copy_bytes": n, "copies": 3}))
 
 
 FWD_STAMPS = ((0, "workgroup starts"), (1, "tile moments in registers (all rows arrived)"), (2, "tile reduced, records published"),
@@ -862,6 +915,128 @@ def torch_gpu_leg(names, device, steps, warmup):
                     "tensors, eager; context only", "us_per_call": out}
 
 
+def counter_bytes_per_config(csv_path, plan, counter):
+    """{config: {"fwd": bytes, "bwd": bytes}} (medians over the calls) from the counter_collection CSV of a
+    `rocprofv3 --pmc <counter>` run of `bench.py --counter-workload`, whose JSON line (`plan`) says how many dispatches
+    each configuration's forward and backward are.  The unit is calibrated on the plain copies the workload starts with."""
+    import collections
+    import csv
+
+    per_dispatch = collections.OrderedDict()
+    with open(csv_path) as f:
+        for r in csv.DictReader(f):
+            # (kernels on _Float16 come out of the profiler with their names still mangled: _ZN2gn...)
+            if ("gn::" not in r["Kernel_Name"] and not r["Kernel_Name"].startswith("_ZN2gn")) or r["Counter_Name"] != counter:
+                continue
+            key = int(r["Dispatch_Id"])
+            name, val = per_dispatch.get(key, (r["Kernel_Name"], 0.0))
+            per_dispatch[key] = (name, val + float(r["Counter_Value"]))
+    seq = [per_dispatch[k] for k in sorted(per_dispatch)]
+    copies = [v for n, v in seq[:plan["copies"]]]
+    assert all("copy_kernel" in n for n, _ in seq[:plan["copies"]]), "the workload does not start with its plain copies"
+    unit = plan["copy_bytes"] / statistics.median(copies)  # bytes per counter unit
+    segments = []  # one per configuration: the dispatches between two marker copies
+    for name, val in seq[plan["copies"]:]:
+        if "copy_kernel" in name:
+            segments.append([])
+        else:
+            segments[-1].append(val)
+    assert len(segments) == len(plan["counter_workload"]), "markers in the counter file do not match the workload's configurations"
+    out = {}
+    for c, seg in zip(plan["counter_workload"], segments):
+        per_call = c["fwd_dispatches"] + c["bwd_dispatches"]
+        assert len(seg) % per_call == 0 and len(seg) >= 3 * per_call, (c["name"], len(seg), per_call)
+        fwd, bwd = [], []
+        for pos in range(0, len(seg), per_call):
+            fwd.append(sum(seg[pos:pos + c["fwd_dispatches"]]))
+            if c["bwd_dispatches"]:
+                bwd.append(sum(seg[pos + c["fwd_dispatches"]:pos + per_call]))
+        out[c["name"]] = {"fwd": statistics.median(fwd) * unit, "bwd": statistics.median(bwd) * unit if bwd else None}
+    return out, unit
+
+
+def results_table(args, device):
+    """The per-configuration result table: us per call, algorithmic GB/s and fraction of the 8 TB/s peak, counter
+    traffic against the algorithmic bytes, the plain copy of the same size, torch's CPU time, and the parity errors
+    observed by tests/test_gpu_parity.py::test_config_parity next to their bars."""
+    import torch
+    import workloads as configs
+
+    names = list(configs.ALL_NAMES)
+    plan = json.loads([ln for ln in open(args.pmc_plan).read().splitlines() if ln.startswith('{"counter_workload"')][-1])
+    fetch, fu = counter_bytes_per_config(args.pmc_fetch, plan, "FETCH_SIZE")
+    write, wu = counter_bytes_per_config(args.pmc_write, plan, "WRITE_SIZE")
+    inst = {c["name"]: c for c in plan["counter_workload"]}
+    errs = {}
+    if args.parity_log:
+        for ln in open(args.parity_log):
+            r = json.loads(ln)
+            if r["family"] == "resident":
+                errs[r["config"]] = r["observed"]
+    cpu = cpu_baseline(names, args.cpu_seconds)
+    steps = max(20, args.steps // 2)
+    print("Per-configuration results on one MI355X: every named configuration, forward and backward through the C ABI, eager launches,")
+    print("each configuration alone in a loop on the same buffers (warm); inputs resident in HBM.")
+    print()
+    print("commands (each rocprofv3 run from /tmp with TMPDIR=/tmp; one counter per run):")
+    print("  GNNHWC_PARITY_LOG=<errors.jsonl> python -m pytest tests/test_gpu_parity.py -m gpu -k test_config_parity")
+    print("  rocprofv3 --pmc FETCH_SIZE --output-format csv -d <fetch> -o p -- python3 bench.py --counter-workload --workload all > <plan.log>")
+    print("  rocprofv3 --pmc WRITE_SIZE --output-format csv -d <write> -o p -- python3 bench.py --counter-workload --workload all")
+    print("  python3 bench.py --results-table --pmc-plan <plan.log> --pmc-fetch <fetch>/p_counter_collection.csv \\")
+    print("          --pmc-write <write>/p_counter_collection.csv --parity-log <errors.jsonl>")
+    print()
+    print("columns: us per call (median of 5 timed loops of %d calls); GB/s = algorithmic bytes (2 S forward, 3 S backward) / time of forward + backward;" % steps)
+    print("  %peak = that / 8000 GB/s; traffic = FETCH_SIZE + WRITE_SIZE of all launches of the call, calibrated on a 256 MiB plain copy")
+    print("  (1 FETCH_SIZE unit = %.1f bytes, 1 WRITE_SIZE unit = %.1f bytes), ratio = traffic / algorithmic bytes; copy us = the library's plain" % (fu, wu))
+    print("  copy kernel reading and writing one tensor of the same size (2 S); cpu us = torch.nn.functional.group_norm + activation (+ autograd)")
+    print("  on %d host threads, same tensors; err = max |ours - truth| / (|truth| + rms(truth)) against the float64 oracle, observed / bar" % cpu["cores"])
+    print("  (float32: bar 1e-5 and also the pure relative error over |truth| >= rms, in brackets; 16-bit: bar = torch's own error in that type + 2 %).")
+    print("  kernel = what the library launched (rows per lane of the register tile, x window rows, two-level exchange, launches per call).")
+    print()
+    hdr = "%-20s %-5s %-22s %7s %7s %8s %7s %6s | %7s %6s %7s %6s | %7s %9s | %-34s | %s" % (
+        "config", "dtype", "shape (N,C,spatial) G", "fwd us", "bwd us", "f+b us", "GB/s", "%peak", "fwd MB", "ratio", "bwd MB", "ratio",
+        "copy us", "cpu us", "err y / dx / dw / db (observed/bar)", "kernel fwd ; bwd")
+    print(hdr)
+    for n in names:
+        cfg = configs.CONFIGS[n]
+        S = configs.tensor_bytes(cfg)
+        prob = Problem(cfg, device, 1)
+        r = measure_shape(prob, None, steps, args.warmup, False)
+        fwd_us = r["warm_fwd_us"]
+        bwd_us = r.get("warm_bwd_us")
+        both_us = r.get("warm_fwd_bwd_us", fwd_us)
+        alg = (5 if prob.bwd else 2) * S
+        gbps = alg / (both_us * 1e-6) / 1e9
+        copy_us = 2 * S / copy_ceiling(S, device, steps) / 1e3
+        ft = fetch[n]["fwd"] + write[n]["fwd"]
+        bt = (fetch[n]["bwd"] + write[n]["bwd"]) if prob.bwd else None
+        e = errs.get(n, {})
+
+        def cell(k):
+            if k not in e:
+                return "-"
+            v = e[k]
+            extra = "[%.0e]" % v["rel"] if cfg.dtype in ("fp32", "fp64") else ""
+            return "%.1e%s/%.1e" % (v["err"], extra, v["bar"])
+
+        print("%-20s %-5s %-22s %7.2f %7s %8.2f %7.0f %6.1f | %7.1f %6.3f %7s %6s | %7.2f %9.0f | %-34s | %s ; %s" % (
+            n, cfg.dtype, "%s G%d %s" % ("x".join(str(v) for v in cfg.shape), cfg.G, cfg.act), fwd_us,
+            "%.2f" % bwd_us if bwd_us else "-", both_us, gbps, 100 * gbps / HBM_PEAK_GBPS, ft / 1e6, ft / (2 * S),
+            "%.1f" % (bt / 1e6) if bt else "-", "%.3f" % (bt / (3 * S)) if bt else "-", copy_us, cpu["us_per_call"][n],
+            " ".join(cell(k) for k in ("y", "dx", "dw", "db")), inst[n]["fwd_instance"], inst[n]["bwd_instance"] or "-"))
+        sys.stdout.flush()
+        del prob
+        torch.cuda.empty_cache()
+    print()
+    print("machine-readable traffic per launch for bench.py (roofline.traffic), single-launch kernels only:")
+    for n in names:
+        c = inst[n]
+        if c["fwd_dispatches"] == 1 and c["fwd_instance"].startswith("fused"):
+            print("TRAFFIC %s fused_fwd %.0f %.0f %s" % (n, fetch[n]["fwd"], write[n]["fwd"], c["fwd_instance"]))
+        if c["bwd_dispatches"] == 1 and c["bwd_instance"] and c["bwd_instance"].startswith("fused"):
+            print("TRAFFIC %s fused_bwd %.0f %.0f %s" % (n, fetch[n]["bwd"], write[n]["bwd"], c["bwd_instance"]))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -885,6 +1060,9 @@ def main():
     if args.code_placement_child >= 0:
         code_placement_child(list(configs.SD_UNET_SWEEP) if args.workload == "sd_unet" else [args.workload], device,
                              args.code_placement_child)
+        return
+    if args.results_table:
+        results_table(args, device)
         return
     if args.switch_cost:
         switch_cost(list(configs.SD_UNET_SWEEP) if args.workload == "sd_unet" else
@@ -940,7 +1118,8 @@ def main():
     dom_bytes = launch_bytes(dom_shape, dominant)
     achieved = dom_bytes / (dom_us * 1e-6) / 1e9
     traffic = recorded_traffic()
-    tr = traffic.get((dom_shape, dominant))
+    by_name = {p.cfg.name: p for p in probs}
+    tr, tr_why = traffic_of(traffic, by_name[dom_shape], dominant)
     roofline = {
         "bound": "hbm",
         "kernel": dominant,
@@ -949,8 +1128,10 @@ def main():
         "peak": HBM_PEAK_GBPS,
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBPS, 4),
-        "traffic": round(tr[0] + tr[1]) if tr else None,
-        "traffic_source": "profiles/hbm_traffic_sd_unet.txt (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, copy-calibrated)" if tr else None,
+        "traffic": round(tr) if tr else None,
+        "traffic_source": ("profiles/results_all_configs.txt (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, copy-calibrated; taken on "
+                           "the kernel instance this run launches: %s)" % by_name[dom_shape].instance("bwd" if "bwd" in dominant else "fwd")
+                           if tr else tr_why),
         "bytes_per_launch": dom_bytes,
         "mean_launch_us": round(dom_us, 3),
         "share_of_step": round(step_us[(dom_shape, dominant)] / total_us, 4),
@@ -958,7 +1139,7 @@ def main():
         "kernels": {n: {k: {"us": round(us, 3), "launches_per_call": per_call, "alg_bytes": launch_bytes(n, k),
                             "frac": round(launch_bytes(n, k) / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
                             "share_of_step": round(step_us[(n, k)] / total_us, 4),
-                            "traffic": (round(sum(traffic[(n, k)])) if (n, k) in traffic else None)}
+                            "traffic": (lambda t: round(t) if t else None)(traffic_of(traffic, by_name[n], k)[0])}
                         for k, (us, per_call) in kinds.items()} for n, kinds in prof.items()},
     }
 

@@ -203,6 +203,7 @@ template <typename PT, int ACT, int NV, int ADD> bool try_resident_fwd_nv(const 
     k.p = pb;
     launch(ADD != kAddNone ? kKindFusedFwdAdd : kKindFusedFwd, r.sync.two_level ? kernel_two : kernel_all, tile_grid(pb, 0),
            dim3(kBlock), a.stream, k);
+    note_resident_launch(ADD != kAddNone ? kKindFusedFwdAdd : kKindFusedFwd, NV, 0, r.sync.two_level, batches, pb.nblocks);
   }
   return true;
 }
@@ -298,6 +299,7 @@ template <typename PT, int ACT, int NV, int XW = 0> bool try_resident_bwd_nv(con
     k.sdtype = a.sdtype;
     k.p = pb;
     launch(kKindFusedBwd, r.sync.two_level ? kernel_two : kernel_all, tile_grid(pb, 0), dim3(kBlock), a.stream, k);
+    note_resident_launch(kKindFusedBwd, NV, XW, r.sync.two_level, batches, pb.nblocks);
   }
   return true;
 }
@@ -339,6 +341,7 @@ bool try_resident_bwd(const BwdArgs &a) {
 #if GN_PART_FWD
 template <int VEC> hipError_t fwd_impl(const FwdArgs &a) {
   if (VEC != 1 && !a.streaming_only && try_resident_fwd(a)) return hipGetLastError();
+  note_streaming_call();
   if (a.has_add()) {
     // multi-launch form: materialise the sum (in sum_out, or in y when the caller does not want it), then
     // normalise it from there (in place when it sits in y)
@@ -424,6 +427,7 @@ template <typename PT, int VEC> void bwd_act(const BwdArgs &a) {
 }
 template <int VEC> hipError_t bwd_impl(const BwdArgs &a) {
   if (VEC != 1 && try_resident_bwd(a)) return hipGetLastError();
+  note_streaming_call();
   if (a.pdtype == GN_INST_DTYPE) bwd_act<elem_t, VEC>(a);
   else bwd_act<wide_param_t, VEC>(a);
   return hipGetLastError();

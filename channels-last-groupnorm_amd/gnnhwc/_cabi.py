@@ -39,6 +39,7 @@ SYMBOLS = (
     "gnnhwc_resident_status",
     "gnnhwc_debug_read_trace",
     "gnnhwc_debug_plan",
+    "gnnhwc_debug_last_launch",
 )
 
 
@@ -93,6 +94,8 @@ def _load():
     lib.gnnhwc_debug_copy.restype = ci
     lib.gnnhwc_debug_plan.argtypes = [i64, i64, i64, i64, ci, ci, ci, ctypes.POINTER(i64)]
     lib.gnnhwc_debug_plan.restype = ci
+    lib.gnnhwc_debug_last_launch.argtypes = [ctypes.POINTER(i64)]
+    lib.gnnhwc_debug_last_launch.restype = ci
     lib.gnnhwc_kernel_kind_name.argtypes = [ci]
     lib.gnnhwc_kernel_kind_name.restype = ctypes.c_char_p
     return lib
@@ -112,6 +115,16 @@ def check(rc, what):
 
 def kernel_kind_names():
     return [lib.gnnhwc_kernel_kind_name(k).decode() for k in range(NUM_KERNEL_KINDS)]
+
+
+def last_launch():
+    """What the calling thread's most recent forward / backward call launched: e.g. 'fused_bwd rows=22 window=0 two_level=0
+    launches=1' for a single-launch kernel, 'multi-launch' for the streaming kernels."""
+    out = (ctypes.c_int64 * 6)()
+    check(lib.gnnhwc_debug_last_launch(out), "gnnhwc_debug_last_launch")
+    if out[0] < 0:
+        return "multi-launch"
+    return "%s rows=%d window=%d two_level=%d launches=%d" % (kernel_kind_names()[out[0]], out[1], out[2], out[3], out[4])
 
 
 def set_resident(on):
