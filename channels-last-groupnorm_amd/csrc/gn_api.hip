@@ -390,14 +390,16 @@ constexpr int kDefaultSpinLimit = 1 << 10;
 std::atomic<int> g_spin_limit{kDefaultSpinLimit};
 int resident_spin_limit() { return g_spin_limit.load(std::memory_order_relaxed); }
 
-thread_local int64_t g_last_launch[6] = {-1, 0, 0, 0, 0, 0};
-void note_resident_launch(int kind, int rows_per_lane, int window_rows, int two_level, int launches, int64_t workgroups) {
+thread_local int64_t g_last_launch[7] = {-1, 0, 0, 0, 0, 0, 0};
+void note_resident_launch(int kind, int rows_per_lane, int window_rows, int parked_rows, int two_level, int launches,
+                          int64_t workgroups) {
   g_last_launch[0] = kind;
   g_last_launch[1] = rows_per_lane;
   g_last_launch[2] = window_rows;
   g_last_launch[3] = two_level;
   g_last_launch[4] = launches;
   g_last_launch[5] = workgroups;
+  g_last_launch[6] = parked_rows;
 }
 void note_streaming_call() { g_last_launch[0] = -1; }
 bool cooperative_launches() {
@@ -698,7 +700,7 @@ int gnnhwc_debug_read_trace(unsigned long long *out, int64_t count) {
 
 int gnnhwc_debug_last_launch(int64_t *out) {
   if (!out) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "null output array");
-  for (int i = 0; i < 6; ++i) out[i] = g_last_launch[i];
+  for (int i = 0; i < 7; ++i) out[i] = g_last_launch[i];
   return GNNHWC_OK;
 }
 

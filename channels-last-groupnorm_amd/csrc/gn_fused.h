@@ -986,6 +986,9 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
 // through a window of XW rows, twice: once for the sums and once, in the opposite direction (so that the window's
 // last rows serve both passes), for dx.  That form holds a tensor half again as large at the price of reading
 // (NV - XW) / NV of x a second time: 4 - XW / NV tensors of traffic, against the 5 of the multi-launch backward.
+// XL > 0 (with XW > 0): the first XL rows of x, which the second pass reaches last, are parked in LDS when the first
+// pass is done with them (16 bytes per lane and row: XL x 4 KB per workgroup, LDS that the register-bound occupancy of
+// these kernels leaves idle) and read back from there: only NV - XW - XL rows are read from memory a second time.
 constexpr int fused_bwd_waves(int nv, int xw) {
   return xw > 0 ? (nv <= 24 ? 3 : 2) : (nv <= 4 ? 4 : nv <= 8 ? 3 : nv <= 22 ? 2 : 1);
 }
@@ -1003,7 +1006,10 @@ struct FusedBwdParams {
   int sdtype, pad_;
   Plan p;
 };
-template <typename T, typename PT, int VEC, int ACT, int NV, bool TWO_LEVEL, int XW = 0>
+// Statistics slots in LDS of a backward kernel: one per group of the chunk.  The kernels with parked rows need their LDS
+// for those and serve chunks of at most kBlock channels (the host checks), hence at most kBlock groups.
+constexpr int fused_bwd_stat_slots(int vec, int xl) { return xl > 0 ? kBlock : kBlock * vec; }
+template <typename T, typename PT, int VEC, int ACT, int NV, bool TWO_LEVEL, int XW = 0, int XL = 0>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bwd_waves(NV, XW)))) void fused_bwd_kernel(
     const FusedBwdParams args) {
   using A = acc_t<T>;
@@ -1017,8 +1023,10 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
   const SyncArea sync = resident_epoch(args.sync);
   __shared__ A sm1[kBlock * VEC];
   __shared__ A sm2[kBlock * VEC];
-  __shared__ A sm_mu[kBlock * VEC];
-  __shared__ A sm_rs[kBlock * VEC];
+  __shared__ A sm_mu[fused_bwd_stat_slots(VEC, XL)];
+  __shared__ A sm_rs[fused_bwd_stat_slots(VEC, XL)];
+  __shared__ typename LV::raw_t parked[XL > 0 ? XL : 1][kBlock];  // rows 0 .. XL - 1 of x between the two passes
+  static_assert(XL == 0 || (XW > 0 && XW + XL <= NV), "parked rows lie below the window's last position");
   __shared__ RecoveryLds recovery;
   if (threadIdx.x == 0) {  // (several barriers lie between this and the first lane that may set either)
     recovery.late = 0;
@@ -1140,6 +1148,9 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
 #pragma unroll
           for (int j = 0; j < VEC; ++j) { pin(s1[j]); pin(s2[j]); }
           pin(bd[u]);  // packed here and now (the conversion otherwise sinks towards the dx phase, g' staying unpacked)
+          if constexpr (XL > 0) {
+            if (u < XL) parked[u][threadIdx.x] = bx[u % NX];
+          }
           if (u + XW < NV) {
             issue_order_fence();  // not before the rows ahead of it are consumed: the slot is the register budget
             bx[u % NX] = LV::load(tile_row(x, t1, u + XW));  // the slot's next row
@@ -1325,14 +1336,21 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
       for (int k = 0; k < NV; ++k) {
         const int u = NV - 1 - k;
         A vx[VEC], vd[VEC];
-        pin(bx[u % NX]);
+        if (XL > 0 && u < XL) {
+          // (a parked row: written and read by the same lane, no barrier needed)
+          typename LV::raw_t back = parked[u][threadIdx.x];
+          pin(back);
+          LV::unpack(back, vx);
+        } else {
+          pin(bx[u % NX]);
+          LV::unpack(bx[u % NX], vx);
+        }
         pin(bd[u]);
-        LV::unpack(bx[u % NX], vx);
         LV::unpack(bd[u], vd);  // g'
 #pragma unroll
         for (int j = 0; j < VEC; ++j) vd[j] = sa[j] * vd[j] + (c1[j] * vx[j] + c2[j]);
         if (u < rows) store_streaming<LV>((T *)tile_row(dx, t2, u), LV::pack(vd));
-        if (u >= XW) {
+        if (u >= XW && u - XW >= XL) {
           issue_order_fence();
           bx[u % NX] = LV::load(tile_row(x, t2, u - XW));
         }

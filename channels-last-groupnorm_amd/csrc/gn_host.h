@@ -165,8 +165,10 @@ class ResidentOrder {
   bool locked_;
 };
 // Which single-launch kernel the calling thread's most recent call used (gnnhwc_debug_last_launch): rows per lane, rows of
-// the x window (0: none), two-level exchange, launches the call was cut into, workgroups of the last launch.
-void note_resident_launch(int kind, int rows_per_lane, int window_rows, int two_level, int launches, int64_t workgroups);
+// the x window (0: none), rows of x parked in LDS, two-level exchange, launches the call was cut into, workgroups of the
+// last launch.
+void note_resident_launch(int kind, int rows_per_lane, int window_rows, int parked_rows, int two_level, int launches,
+                          int64_t workgroups);
 void note_streaming_call();
 bool resident_enabled();
 // Device buffer for in-kernel timestamps when GNNHWC_TRACE=1, else null.

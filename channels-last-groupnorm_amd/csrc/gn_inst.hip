@@ -203,7 +203,7 @@ template <typename PT, int ACT, int NV, int ADD> bool try_resident_fwd_nv(const 
     k.p = pb;
     launch(ADD != kAddNone ? kKindFusedFwdAdd : kKindFusedFwd, r.sync.two_level ? kernel_two : kernel_all, tile_grid(pb, 0),
            dim3(kBlock), a.stream, k);
-    note_resident_launch(ADD != kAddNone ? kKindFusedFwdAdd : kKindFusedFwd, NV, 0, r.sync.two_level, batches, pb.nblocks);
+    note_resident_launch(ADD != kAddNone ? kKindFusedFwdAdd : kKindFusedFwd, NV, 0, 0, r.sync.two_level, batches, pb.nblocks);
   }
   return true;
 }
@@ -254,10 +254,12 @@ bool try_resident_fwd(const FwdArgs &a) {
 #endif  // !GN_PART_BWD
 
 #if GN_PART_BWD
-template <typename PT, int ACT, int NV, int XW = 0> bool try_resident_bwd_nv(const BwdArgs &a, int batches) {
+template <typename PT, int ACT, int NV, int XW = 0, int XL = 0> bool try_resident_bwd_nv(const BwdArgs &a, int batches) {
   if (NV < resident_min_rows()) return false;
-  auto kernel_all = fused_bwd_kernel<elem_t, PT, kVec, ACT, NV, false, XW>;
-  auto kernel_two = fused_bwd_kernel<elem_t, PT, kVec, ACT, NV, true, XW>;
+  // (kernels that park rows of x in LDS have statistics slots for chunks of at most kBlock channels)
+  if (XL > 0 && a.plan.lpr * a.plan.vec > kBlock) return false;
+  auto kernel_all = fused_bwd_kernel<elem_t, PT, kVec, ACT, NV, false, XW, XL>;
+  auto kernel_two = fused_bwd_kernel<elem_t, PT, kVec, ACT, NV, true, XW, XL>;
   static const int slots = std::min(resident_slots(kernel_all), resident_slots(kernel_two));
   const int64_t per = (a.plan.N + batches - 1) / batches;
   Plan p;
@@ -299,7 +301,7 @@ template <typename PT, int ACT, int NV, int XW = 0> bool try_resident_bwd_nv(con
     k.sdtype = a.sdtype;
     k.p = pb;
     launch(kKindFusedBwd, r.sync.two_level ? kernel_two : kernel_all, tile_grid(pb, 0), dim3(kBlock), a.stream, k);
-    note_resident_launch(kKindFusedBwd, NV, XW, r.sync.two_level, batches, pb.nblocks);
+    note_resident_launch(kKindFusedBwd, NV, XW, XL, r.sync.two_level, batches, pb.nblocks);
   }
   return true;
 }
@@ -312,9 +314,11 @@ template <typename PT, int ACT> bool try_resident_bwd_act(const BwdArgs &a) {
       return true;
     // too large for two tiles in registers: the form that keeps g' and reads most of x twice, before the tensor is cut
     // into more launches (measured on bf16 (N, 320, 128, 128): 32.6 against 39.3 us at N = 5, 37.2 against 43.4 at N = 6)
-    // (window: what the registers leave beside 32 rows of g', 16 rows for 16-bit data)
+    // (window: what the registers leave beside 32 rows of g', 16 rows for 16-bit data; parked: the rows of x that two
+    // workgroups per CU can keep in LDS beside their reduction arrays, 14 x 4 KB for 16-bit data, 16 x 4 KB for float)
     constexpr int window = sizeof(elem_t) == 2 ? 16 : 12;
-    if (try_resident_bwd_nv<PT, ACT, 32, window>(a, b) || try_resident_bwd_nv<PT, ACT, 36, 8>(a, b)) return true;
+    constexpr int parked = sizeof(elem_t) == 2 ? 14 : 16;
+    if (try_resident_bwd_nv<PT, ACT, 32, window, parked>(a, b) || try_resident_bwd_nv<PT, ACT, 36, 8, parked>(a, b)) return true;
   }
   return false;
 }

@@ -118,13 +118,13 @@ def kernel_kind_names():
 
 
 def last_launch():
-    """What the calling thread's most recent forward / backward call launched: e.g. 'fused_bwd rows=22 window=0 two_level=0
-    launches=1' for a single-launch kernel, 'multi-launch' for the streaming kernels."""
-    out = (ctypes.c_int64 * 6)()
+    """What the calling thread's most recent forward / backward call launched: e.g. 'fused_bwd rows=22 window=0 parked=0
+    two_level=0 launches=1' for a single-launch kernel, 'multi-launch' for the streaming kernels."""
+    out = (ctypes.c_int64 * 7)()
     check(lib.gnnhwc_debug_last_launch(out), "gnnhwc_debug_last_launch")
     if out[0] < 0:
         return "multi-launch"
-    return "%s rows=%d window=%d two_level=%d launches=%d" % (kernel_kind_names()[out[0]], out[1], out[2], out[3], out[4])
+    return "%s rows=%d window=%d parked=%d two_level=%d launches=%d" % (kernel_kind_names()[out[0]], out[1], out[2], out[6], out[3], out[4])
 
 
 def set_resident(on):

@@ -264,12 +264,13 @@ int gnnhwc_debug_set_spin_limit(int polls);
 
 /*
  * Which kernels the calling thread's most recent gnnhwc_fwd / _fwd_add / _fwd_cast / gnnhwc_bwd call launched (no
- * counterpart in the reference; for benchmarks and tests that must know what they measured).  out[6] receives: the
+ * counterpart in the reference; for benchmarks and tests that must know what they measured).  out[7] receives: the
  * kernel kind (6, 7 or 10: a single-launch kernel; -1: the multi-launch kernels), rows per lane of the register tile,
  * rows of the x window of a backward that keeps g' only (0: x is kept too), 1 if the two-level exchange was used,
- * the number of launches the call was cut into (over groups of samples), workgroups of the last of them.
+ * the number of launches the call was cut into (over groups of samples), workgroups of the last of them, rows of x
+ * that backward parks in LDS between its two passes.
  */
-int gnnhwc_debug_last_launch(int64_t *out /* [6] */);
+int gnnhwc_debug_last_launch(int64_t *out /* [7] */);
 
 /*
  * Plain device-to-device copy of `bytes` (a multiple of 16; 16-byte aligned pointers) by a kernel with the
