@@ -802,6 +802,33 @@ def cast_table(names, device, steps, warmup):
             r[key + "_us"] = round(t * 1e6, 3)
             r[key + "_gbps"] = round(1.5 * p.S / t / 1e9, 1)  # algorithmic bytes of the FUSED form / time
         r["speedup"] = round(r["unfused_us"] / r["fused_us"], 3)
+        # the backward that follows: the gradient of y arrives as bfloat16; read as it is (gnnhwc_bwd_cast: x S, dy S / 2,
+        # dx S) against a widening pass (1.5 S more) followed by gnnhwc_bwd
+        if p.bwd:
+            dy16 = torch.randn(x.shape, device=device).to(torch.bfloat16)
+            dyf = torch.empty_like(x)
+
+            def bwd_fused():
+                rc = p.lib.gnnhwc_bwd_cast(dy16.data_ptr(), x.data_ptr(), p.w.data_ptr(), p.b.data_ptr(), p.mean.data_ptr(),
+                                           p.rstd.data_ptr(), b["dx"].data_ptr(), p.dw.data_ptr(), p.db.data_ptr(), p.N, p.R, p.C,
+                                           p.G, p.act, p.dt, p.dt, p.sdt, 3, p.ws_b.data_ptr(), p.ws_b.numel(), stream_of())
+                if rc != 0:
+                    raise RuntimeError(p.lib.gnnhwc_last_error().decode())
+
+            def bwd_unfused():
+                dyf.copy_(dy16)
+                rc = p.lib.gnnhwc_bwd(dyf.data_ptr(), x.data_ptr(), p.w.data_ptr(), p.b.data_ptr(), p.mean.data_ptr(),
+                                      p.rstd.data_ptr(), b["dx"].data_ptr(), p.dw.data_ptr(), p.db.data_ptr(), p.N, p.R, p.C, p.G,
+                                      p.act, p.dt, p.dt, p.sdt, p.ws_b.data_ptr(), p.ws_b.numel(), stream_of())
+                if rc != 0:
+                    raise RuntimeError(p.lib.gnnhwc_last_error().decode())
+
+            fused()  # (mean / rstd of this x)
+            for key, fn in (("bwd_fused", bwd_fused), ("bwd_unfused", bwd_unfused)):
+                t = min(time_region(fn, steps, warmup, False) for _ in range(3)) / steps
+                r[key + "_us"] = round(t * 1e6, 3)
+                r[key + "_gbps"] = round(2.5 * p.S / t / 1e9, 1)  # algorithmic bytes of the FUSED form / time
+            r["bwd_speedup"] = round(r["bwd_unfused_us"] / r["bwd_fused_us"], 3)
         out[n + "_fp32"] = r
         del p
         torch.cuda.empty_cache()

@@ -600,13 +600,16 @@ int gnnhwc_fwd_add(const void *x, const void *residual, const void *channel_bias
                  workspace_bytes, stream);
 }
 
-int gnnhwc_bwd(const void *dy, const void *x, const void *weight, const void *bias, const void *mean, const void *rstd,
-               void *dx, void *dweight, void *dbias, int64_t N, int64_t R, int64_t C, int64_t G, int act, int dtype,
-               int param_dtype, int stats_dtype, void *workspace, size_t workspace_bytes, void *stream) {
+static int backward(const void *dy, const void *x, const void *weight, const void *bias, const void *mean, const void *rstd,
+                    void *dx, void *dweight, void *dbias, int64_t N, int64_t R, int64_t C, int64_t G, int act, int dtype,
+                    int param_dtype, int stats_dtype, int dy_dtype, void *workspace, size_t workspace_bytes, void *stream) {
   int rc = check_shape(N, R, C, G, dtype);
   if (rc != GNNHWC_OK) return rc;
   rc = check_dtypes(dtype, param_dtype, stats_dtype);
   if (rc != GNNHWC_OK) return rc;
+  if (dy_dtype != dtype && !(dtype == GN_F32 && (dy_dtype == GN_F16 || dy_dtype == GN_BF16)))
+    return fail(GNNHWC_ERR_INVALID_ARGUMENT, "dy_dtype %d with dtype %d: dy is read in dtype, or as F16 / BF16 for F32 data",
+                dy_dtype, dtype);
   if (act < GN_ACT_IDENTITY || act > GN_ACT_GELU_TANH)
     return fail(GNNHWC_ERR_INVALID_ARGUMENT, "unknown activation code %d", act);
   if (N == 0 || R == 0) {
@@ -625,8 +628,10 @@ int gnnhwc_bwd(const void *dy, const void *x, const void *weight, const void *bi
     return fail(GNNHWC_ERR_WORKSPACE, "backward workspace must be 16-byte aligned and at least %zu bytes (got %p, %zu bytes)",
                 need, workspace, workspace_bytes);
   const int vec = 16 / elem_size(dtype);
+  if (dy_dtype != dtype && dx == dy) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "dx of another type than dy cannot replace dy in place");
   const bool vector_ok = C % vec == 0 && aligned16(x) && aligned16(dy) && aligned16(dx);
   BwdArgs a;
+  a.dydtype = dy_dtype;
   a.dy = dy; a.x = x; a.w = weight; a.b = bias; a.mean = mean; a.rstd = rstd;
   a.dx = dx; a.dw = dweight; a.db = dbias;
   a.act = act; a.pdtype = param_dtype; a.sdtype = stats_dtype;
@@ -643,6 +648,21 @@ int gnnhwc_bwd(const void *dy, const void *x, const void *weight, const void *bi
   }
   if (e != hipSuccess) return fail(GNNHWC_ERR_LAUNCH, "backward launch failed: %s", hipGetErrorString(e));
   return GNNHWC_OK;
+}
+
+int gnnhwc_bwd(const void *dy, const void *x, const void *weight, const void *bias, const void *mean, const void *rstd,
+               void *dx, void *dweight, void *dbias, int64_t N, int64_t R, int64_t C, int64_t G, int act, int dtype,
+               int param_dtype, int stats_dtype, void *workspace, size_t workspace_bytes, void *stream) {
+  return backward(dy, x, weight, bias, mean, rstd, dx, dweight, dbias, N, R, C, G, act, dtype, param_dtype, stats_dtype, dtype,
+                  workspace, workspace_bytes, stream);
+}
+
+int gnnhwc_bwd_cast(const void *dy, const void *x, const void *weight, const void *bias, const void *mean, const void *rstd,
+                    void *dx, void *dweight, void *dbias, int64_t N, int64_t R, int64_t C, int64_t G, int act, int dtype,
+                    int param_dtype, int stats_dtype, int dy_dtype, void *workspace, size_t workspace_bytes, void *stream) {
+  if (dy_dtype < GN_F32 || dy_dtype > GN_BF16) return fail(GNNHWC_ERR_INVALID_ARGUMENT, "unknown dy_dtype code %d", dy_dtype);
+  return backward(dy, x, weight, bias, mean, rstd, dx, dweight, dbias, N, R, C, G, act, dtype, param_dtype, stats_dtype, dy_dtype,
+                  workspace, workspace_bytes, stream);
 }
 
 int gnnhwc_profile_enable(int on) {

@@ -397,10 +397,14 @@ __device__ __forceinline__ void channel_coeffs(const void *w, const void *b, int
 }
 // Backward group record (t, k, g) of the sample at xs / dys: {sum_c gamma_c sum g' x, sum_c gamma_c sum g'} with
 // g' = dy act'(x a_c + b_c), by the whole workgroup.  mu, rs: the group's statistics.
-template <typename T, typename PT, int ACT>
-__device__ __forceinline__ void recompute_bwd_record(const T *xs, const T *dys, const void *w, const void *b, const Plan &p,
-                                                     int t, int k, int g, float mu, float rs, double *scratch, float &va,
-                                                     float &vb) {
+// Pointer to element e of a gradient that is stored in T or (DY16) in a 16-bit type, as a T pointer that load_dy accepts.
+template <typename T, bool DY16> __device__ __forceinline__ const T *dy_at(const T *dy, int64_t e) {
+  return DY16 ? (const T *)((const uint16_t *)dy + e) : dy + e;
+}
+template <typename T, typename PT, int ACT, bool DY16>
+__device__ __forceinline__ void recompute_bwd_record(const T *xs, const T *dys, int dydtype, const void *w, const void *b,
+                                                     const Plan &p, int t, int k, int g, float mu, float rs, double *scratch,
+                                                     float &va, float &vb) {
   using L1 = LaneVec<T, 1>;
   const RecordSpan sp = record_span(p, t, k, g);
   const int nc = sp.c_hi - sp.c_lo;
@@ -410,11 +414,11 @@ __device__ __forceinline__ void recompute_bwd_record(const T *xs, const T *dys, 
   for (int64_t i = threadIdx.x; i < cnt; i += kBlock) {
     const int64_t r = i / nc;
     const int c = sp.c_lo + (int)(i - r * nc);
-    float gamma, a, bb, vx[1], vd[1];
+    float gamma, a, bb, vx[1];
     channel_coeffs<PT>(w, b, c, mu, rs, gamma, a, bb);
     L1::unpack(L1::load(xs + (sp.r0 + r) * p.C + c), vx);
-    L1::unpack(L1::load(dys + (sp.r0 + r) * p.C + c), vd);
-    const float gp = vd[0] * act_bwd<ACT, float>(vx[0] * a + bb);
+    const float vd = load_dy_scalar<T, DY16>(dys, (sp.r0 + r) * p.C + c, dydtype);
+    const float gp = vd * act_bwd<ACT, float>(vx[0] * a + bb);
     ta += (double)gamma * ((double)gp * (double)vx[0]);
     tb += (double)gamma * (double)gp;
   }
@@ -423,19 +427,19 @@ __device__ __forceinline__ void recompute_bwd_record(const T *xs, const T *dys, 
   vb = (float)tb;
 }
 // Backward channel record (tile t, channel c) of the sample at xs / dys: {sum g' x, sum g'} over the tile's rows.
-template <typename T, int ACT>
-__device__ __forceinline__ void recompute_channel_record(const T *xs, const T *dys, const Plan &p, int t, int c, float a, float bb,
-                                                         double *scratch, float &v0, float &v1) {
+template <typename T, int ACT, bool DY16>
+__device__ __forceinline__ void recompute_channel_record(const T *xs, const T *dys, int dydtype, const Plan &p, int t, int c,
+                                                         float a, float bb, double *scratch, float &v0, float &v1) {
   using L1 = LaneVec<T, 1>;
   const int64_t r0 = (int64_t)t * p.tile_rows;
   const int64_t r1 = r0 + p.tile_rows < p.R ? r0 + p.tile_rows : p.R;
   double S1 = 0.0, S2 = 0.0;
 #pragma nounroll
   for (int64_t r = r0 + threadIdx.x; r < r1; r += kBlock) {
-    float vx[1], vd[1];
+    float vx[1];
     L1::unpack(L1::load(xs + r * p.C + c), vx);
-    L1::unpack(L1::load(dys + r * p.C + c), vd);
-    const float gp = vd[0] * act_bwd<ACT, float>(vx[0] * a + bb);
+    const float vd = load_dy_scalar<T, DY16>(dys, r * p.C + c, dydtype);
+    const float gp = vd * act_bwd<ACT, float>(vx[0] * a + bb);
     S1 += (double)gp * (double)vx[0];
     S2 += (double)gp;
   }
@@ -556,9 +560,9 @@ __device__ __forceinline__ void recover_fwd(const T *x, T *y, const SyncArea &sy
 
 // The same for a backward workgroup, up to and including its rows of dx: the group sums of the chunk's groups from the
 // tile records (or from x and dy where they are missing) give the coefficients, then dx row by row from memory.
-template <typename T, typename PT, int VEC, int ACT, bool TWO_LEVEL>
-__device__ __forceinline__ void recover_bwd_dx(const T *x, const T *dy, T *dx, const void *mean, const void *rstd, int sdtype,
-                                               const void *w, const void *b, const SyncArea &sync, const Plan &p,
+template <typename T, typename PT, int VEC, int ACT, bool TWO_LEVEL, bool DY16>
+__device__ __forceinline__ void recover_bwd_dx(const T *x, const T *dy, T *dx, int dydtype, const void *mean, const void *rstd,
+                                               int sdtype, const void *w, const void *b, const SyncArea &sync, const Plan &p,
                                                RecoveryLds &r, const float *sm_mu, const float *sm_rs, float *sm_k1,
                                                float *sm_k2) {
   using LV = LaneVec<T, VEC>;
@@ -581,7 +585,7 @@ __device__ __forceinline__ void recover_bwd_dx(const T *x, const T *dy, T *dx, c
           tb += rbv;
         },
         [&](int t, int k, float &v0, float &v1) {
-          recompute_bwd_record<T, PT, ACT>(x + sample, dy + sample, w, b, p, t, k, g, mu, rs, r.sums, v0, v1);
+          recompute_bwd_record<T, PT, ACT, DY16>(x + sample, dy_at<T, DY16>(dy, sample), dydtype, w, b, p, t, k, g, mu, rs, r.sums, v0, v1);
         });
     const double sc = 1.0 / ((double)p.D * (double)p.R);
     const double k1 = ((double)mu * tb - ta) * sc * (double)rs * (double)rs * (double)rs;
@@ -604,7 +608,7 @@ __device__ __forceinline__ void recover_bwd_dx(const T *x, const T *dy, T *dx, c
     for (int u = 0; u < l.rows; ++u) {
       float vx[VEC], vd[VEC];
       LV::unpack(LV::load(x + off + (int64_t)u * step), vx);
-      LV::unpack(LV::load(dy + off + (int64_t)u * step), vd);
+      unpack_dy<T, VEC, DY16>(load_dy<T, VEC, DY16>(dy, off + (int64_t)u * step), vd, dydtype);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) vd[j] = vd[j] * act_bwd<ACT, float>(vx[j] * sa[j] + sb[j]);
       // (g' passes through T as on the fast path, where it waits in registers in packed form)
@@ -620,8 +624,8 @@ __device__ __forceinline__ void recover_bwd_dx(const T *x, const T *dy, T *dx, c
 // dgamma / dbeta of the channels this workgroup finishes, after an expired wait of that stage: every channel record
 // of the whole tensor that feeds them is taken as it arrived, or rebuilt from x and dy.  Records of samples before n0
 // were written by launches that have ended.  x / dy point at sample n0.
-template <typename T, typename PT, int ACT>
-__device__ __forceinline__ void recover_bwd_tail(const T *x, const T *dy, const void *w, const void *b, const void *mean_all,
+template <typename T, typename PT, int ACT, bool DY16>
+__device__ __forceinline__ void recover_bwd_tail(const T *x, const T *dy, int dydtype, const void *w, const void *b, const void *mean_all,
                                                  const void *rstd_all, int sdtype, const SyncArea &sync, const Plan &p,
                                                  RecoveryLds &r, int64_t n0, int64_t n_all, void *dw, void *db) {
   const int salt = opaque_zero();
@@ -655,7 +659,7 @@ __device__ __forceinline__ void recover_bwd_tail(const T *x, const T *dy, const 
             float gamma, a, bb;
             channel_coeffs<PT>(w, b, c, mu, rs, gamma, a, bb);
             const int64_t sample = (int64_t)(nn - n0) * p.R * p.C;
-            recompute_channel_record<T, ACT>(x + sample, dy + sample, p, t, c, a, bb, r.sums, v0, v1);
+            recompute_channel_record<T, ACT, DY16>(x + sample, dy_at<T, DY16>(dy, sample), dydtype, p, t, c, a, bb, r.sums, v0, v1);
             prefer_arrived(sync, rbc, r, slot_of(e), v0, v1);
           }
           t1 += ((double)v0 - (double)mu * (double)v1) * (double)rs;
@@ -1003,13 +1007,14 @@ struct FusedBwdParams {
   void *dw, *db;
   const void *mean_all, *rstd_all;
   int64_t n0, n_all;
-  int sdtype, pad_;
+  int sdtype;
+  int dydtype;  // type dy is stored in: the data type, or for float data GN_F16 / GN_BF16 (kernels instantiated with DY16)
   Plan p;
 };
 // Statistics slots in LDS of a backward kernel: one per group of the chunk.  The kernels with parked rows need their LDS
 // for those and serve chunks of at most kBlock channels (the host checks), hence at most kBlock groups.
 constexpr int fused_bwd_stat_slots(int vec, int xl) { return xl > 0 ? kBlock : kBlock * vec; }
-template <typename T, typename PT, int VEC, int ACT, int NV, bool TWO_LEVEL, int XW = 0, int XL = 0>
+template <typename T, typename PT, int VEC, int ACT, int NV, bool TWO_LEVEL, int XW = 0, int XL = 0, bool DY16 = false>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bwd_waves(NV, XW)))) void fused_bwd_kernel(
     const FusedBwdParams args) {
   using A = acc_t<T>;
@@ -1065,6 +1070,11 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
   auto tile_row = [&](const T *base, const RowTerms &t, int u) {
     return (const T *)((const char *)(base + tile_base) + (t.lane0 + (unsigned)clamp_row(u, t.rows) * t.step));
   };
+  // (a 16-bit gradient beside float data: the same element offsets at half the bytes)
+  auto dy_row = [&](const RowTerms &t, int u) {
+    const unsigned bytes = t.lane0 + (unsigned)clamp_row(u, t.rows) * t.step;
+    return DY16 ? (const T *)((const char *)dy + tile_base * 2 + (bytes >> 1)) : (const T *)((const char *)(dy + tile_base) + bytes);
+  };
   trace_point(sync, 0);
   // the small loads go first: loads return in order, so the statistics and parameters, which the first row's
   // arithmetic needs, must not queue behind the whole tile.  Nothing here is under a branch (idle lanes read valid
@@ -1087,7 +1097,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
     for (int u = 0; u < NV; ++u) {
       const int64_t o = row_offset(u);
       bx[u] = LV::load(x + o);
-      bd[u] = LV::load(dy + o);
+      bd[u] = load_dy<T, VEC, DY16>(dy, o);
     }
   } else {
     // the window of x first (row 0's arithmetic needs it), then all of dy; the rest of x follows row by row below
@@ -1095,7 +1105,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
 #pragma unroll
     for (int u = 0; u < XW; ++u) bx[u] = LV::load(tile_row(x, t0, u));
 #pragma unroll
-    for (int u = 0; u < NV; ++u) bd[u] = LV::load(tile_row(dy, t0, u));
+    for (int u = 0; u < NV; ++u) bd[u] = load_dy<T, VEC, DY16>(dy_row(t0, u), 0);
   }
   commit_chunk_stats<A>(st, l, sm_mu, sm_rs);
   __builtin_amdgcn_s_setprio(2);  // towards the exchange: ahead of wavefronts that are already past theirs
@@ -1124,7 +1134,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
         pin(bx[u % NX]);  // one row at a time: cheap activations otherwise tempt the scheduler into unpacking many
         pin(bd[u]);       // rows ahead, which costs more registers than the tile itself
         LV::unpack(bx[u % NX], vx);
-        LV::unpack(bd[u], vd);
+        unpack_dy<T, VEC, DY16>(bd[u], vd, args.dydtype);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) {
           if constexpr (XW > 0 && VEC >= 4) {
@@ -1288,11 +1298,11 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
     const FusedBwdParams ka = reread_kernel_args<FusedBwdParams>();
     SyncArea ks = ka.sync;
     ks.epoch = epoch;
-    recover_bwd_dx<T, PT, VEC, ACT, TWO_LEVEL>((const T *)ka.x, (const T *)ka.dy, (T *)ka.dx, ka.mean, ka.rstd, ka.sdtype, ka.w, ka.b,
-                                               ks, ka.p, recovery, sm_mu, sm_rs, sm1, sm2);
+    recover_bwd_dx<T, PT, VEC, ACT, TWO_LEVEL, DY16>((const T *)ka.x, (const T *)ka.dy, (T *)ka.dx, ka.dydtype, ka.mean, ka.rstd,
+                                                     ka.sdtype, ka.w, ka.b, ks, ka.p, recovery, sm_mu, sm_rs, sm1, sm2);
     if (blockIdx.z == 0 && (ka.dw || ka.db))
-      recover_bwd_tail<T, PT, ACT>((const T *)ka.x, (const T *)ka.dy, ka.w, ka.b, ka.mean_all, ka.rstd_all, ka.sdtype, ks, ka.p,
-                                   recovery, ka.n0, ka.n_all, ka.dw, ka.db);
+      recover_bwd_tail<T, PT, ACT, DY16>((const T *)ka.x, (const T *)ka.dy, ka.dydtype, ka.w, ka.b, ka.mean_all, ka.rstd_all, ka.sdtype,
+                                         ks, ka.p, recovery, ka.n0, ka.n_all, ka.dw, ka.db);
     return;
   }
   const int tslot = threadIdx.x >> tlg, tsl = threadIdx.x & (TL - 1);
@@ -1413,8 +1423,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
       const FusedBwdParams ka = reread_kernel_args<FusedBwdParams>();
       SyncArea ks = ka.sync;
       ks.epoch = epoch;
-      recover_bwd_tail<T, PT, ACT>((const T *)ka.x, (const T *)ka.dy, ka.w, ka.b, ka.mean_all, ka.rstd_all, ka.sdtype, ks, ka.p,
-                                   recovery, ka.n0, ka.n_all, ka.dw, ka.db);
+      recover_bwd_tail<T, PT, ACT, DY16>((const T *)ka.x, (const T *)ka.dy, ka.dydtype, ka.w, ka.b, ka.mean_all, ka.rstd_all, ka.sdtype,
+                                         ks, ka.p, recovery, ka.n0, ka.n_all, ka.dw, ka.db);
     }
   }
   }

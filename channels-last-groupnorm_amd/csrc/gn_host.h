@@ -49,6 +49,7 @@ struct BwdArgs {
   const void *dy, *x, *w, *b, *mean, *rstd;
   void *dx, *dw, *db;
   int act, pdtype, sdtype;
+  int dydtype;  // type dy is stored in: the data type, or for float data GN_F16 / GN_BF16
   void *ws;
   hipStream_t stream;
   Plan plan;

@@ -254,12 +254,22 @@ bool try_resident_fwd(const FwdArgs &a) {
 #endif  // !GN_PART_BWD
 
 #if GN_PART_BWD
+// dy stored in a 16-bit type while the data are float (only the float instantiation has such kernels)
+constexpr bool kHasDy16 = GN_INST_DTYPE == 0;
+template <typename PT, int ACT, int NV, int XW, int XL, bool DY16> bool try_resident_bwd_one(const BwdArgs &a, int batches);
 template <typename PT, int ACT, int NV, int XW = 0, int XL = 0> bool try_resident_bwd_nv(const BwdArgs &a, int batches) {
+  if (a.dydtype != GN_INST_DTYPE) {
+    if constexpr (kHasDy16) return try_resident_bwd_one<PT, ACT, NV, XW, XL, true>(a, batches);
+    else return false;
+  }
+  return try_resident_bwd_one<PT, ACT, NV, XW, XL, false>(a, batches);
+}
+template <typename PT, int ACT, int NV, int XW, int XL, bool DY16> bool try_resident_bwd_one(const BwdArgs &a, int batches) {
   if (NV < resident_min_rows()) return false;
   // (kernels that park rows of x in LDS have statistics slots for chunks of at most kBlock channels)
   if (XL > 0 && a.plan.lpr * a.plan.vec > kBlock) return false;
-  auto kernel_all = fused_bwd_kernel<elem_t, PT, kVec, ACT, NV, false, XW, XL>;
-  auto kernel_two = fused_bwd_kernel<elem_t, PT, kVec, ACT, NV, true, XW, XL>;
+  auto kernel_all = fused_bwd_kernel<elem_t, PT, kVec, ACT, NV, false, XW, XL, DY16>;
+  auto kernel_two = fused_bwd_kernel<elem_t, PT, kVec, ACT, NV, true, XW, XL, DY16>;
   static const int slots = std::min(resident_slots(kernel_all), resident_slots(kernel_two));
   const int64_t per = (a.plan.N + batches - 1) / batches;
   Plan p;
@@ -285,7 +295,8 @@ template <typename PT, int ACT, int NV, int XW = 0, int XL = 0> bool try_residen
     const bool last = n0 + per >= a.plan.N;
     FusedBwdParams k = {};
     k.x = (const elem_t *)a.x + n0 * sample;
-    k.dy = (const elem_t *)a.dy + n0 * sample;
+    k.dy = (const char *)a.dy + n0 * sample * stat_size(a.dydtype);
+    k.dydtype = a.dydtype;
     k.dx = (elem_t *)a.dx + n0 * sample;
     k.mean = (const char *)a.mean + n0 * a.plan.G * ssz;
     k.rstd = (const char *)a.rstd + n0 * a.plan.G * ssz;
@@ -392,15 +403,15 @@ template <int VEC> hipError_t fwd_impl(const FwdArgs &a) {
 #endif  // GN_PART_FWD
 
 #if GN_PART_BWD
-template <typename PT, int VEC, int ACT> void launch_bwd_act(const BwdArgs &a) {
+template <typename PT, int VEC, int ACT, bool DY16> void launch_bwd_act(const BwdArgs &a) {
   const Plan &p = a.plan;
   const BwdWorkspace ws = bwd_workspace(p);
   A *base = (A *)((char *)a.ws + kWorkspaceHeader);
   A *partC = base + ws.partC, *partG = base + ws.partG, *compactC = base + ws.compactC, *compactG = base + ws.compactG;
   PartialGeo q = producer_geo(p);
   {
-    launch(kKindBwdReduce, (bwd_reduce_kernel<elem_t, PT, VEC, ACT>), tile_grid(p, 0), dim3(kBlock), a.stream,
-                       (const elem_t *)a.x, (const elem_t *)a.dy, a.mean, a.rstd, a.sdtype, a.w, a.b, partC, partG, p);
+    launch(kKindBwdReduce, (bwd_reduce_kernel<elem_t, PT, VEC, ACT, DY16>), tile_grid(p, 0), dim3(kBlock), a.stream,
+                       (const elem_t *)a.x, (const elem_t *)a.dy, a.mean, a.rstd, a.sdtype, a.w, a.b, partC, partG, p, a.dydtype);
   }
   const A *srcC = partC, *srcG = partG;
   if (needs_compaction(p)) {
@@ -415,19 +426,25 @@ template <typename PT, int VEC, int ACT> void launch_bwd_act(const BwdArgs &a) {
     srcG = compactG;
   }
   {
-    launch(kKindBwdDx, (bwd_dx_kernel<elem_t, PT, VEC, ACT>), tile_grid(p, 1), dim3(kBlock), a.stream,
+    launch(kKindBwdDx, (bwd_dx_kernel<elem_t, PT, VEC, ACT, DY16>), tile_grid(p, 1), dim3(kBlock), a.stream,
                        (const elem_t *)a.x, (const elem_t *)a.dy, (elem_t *)a.dx, a.mean, a.rstd, a.sdtype, a.w, a.b, srcC,
-                       srcG, q, a.dw, a.db, p);
+                       srcG, q, a.dw, a.db, p, a.dydtype);
+  }
+}
+template <typename PT, int VEC, bool DY16> void bwd_act_dy(const BwdArgs &a) {
+  switch (a.act) {
+    case GN_ACT_IDENTITY: launch_bwd_act<PT, VEC, GN_ACT_IDENTITY, DY16>(a); break;
+    case GN_ACT_RELU: launch_bwd_act<PT, VEC, GN_ACT_RELU, DY16>(a); break;
+    case GN_ACT_SILU: launch_bwd_act<PT, VEC, GN_ACT_SILU, DY16>(a); break;
+    case GN_ACT_GELU: launch_bwd_act<PT, VEC, GN_ACT_GELU, DY16>(a); break;
+    default: launch_bwd_act<PT, VEC, GN_ACT_GELU_TANH, DY16>(a); break;
   }
 }
 template <typename PT, int VEC> void bwd_act(const BwdArgs &a) {
-  switch (a.act) {
-    case GN_ACT_IDENTITY: launch_bwd_act<PT, VEC, GN_ACT_IDENTITY>(a); break;
-    case GN_ACT_RELU: launch_bwd_act<PT, VEC, GN_ACT_RELU>(a); break;
-    case GN_ACT_SILU: launch_bwd_act<PT, VEC, GN_ACT_SILU>(a); break;
-    case GN_ACT_GELU: launch_bwd_act<PT, VEC, GN_ACT_GELU>(a); break;
-    default: launch_bwd_act<PT, VEC, GN_ACT_GELU_TANH>(a); break;
+  if constexpr (kHasDy16) {
+    if (a.dydtype != GN_INST_DTYPE) return bwd_act_dy<PT, VEC, true>(a);
   }
+  bwd_act_dy<PT, VEC, false>(a);
 }
 template <int VEC> hipError_t bwd_impl(const BwdArgs &a) {
   if (VEC != 1 && try_resident_bwd(a)) return hipGetLastError();

@@ -130,6 +130,52 @@ template <typename PT, typename A> __device__ __forceinline__ void store_param(v
   LaneVec<PT, 1>::store((PT *)p + i, LaneVec<PT, 1>::pack(v));
 }
 
+// The incoming gradient of a backward on float data may be stored in a 16-bit type (DY16; dydtype GN_F16 or GN_BF16: the
+// layer that produced it ran in half precision).  A lane vector of it is 8 bytes, carried in the first half of the raw
+// register vector until it is unpacked; widening happens in registers, no separate pass over dy.
+template <typename T, int VEC, bool DY16>
+__device__ __forceinline__ typename LaneVec<T, VEC>::raw_t load_dy(const T *dy, int64_t e) {
+  if constexpr (!DY16) {
+    return LaneVec<T, VEC>::load(dy + e);
+  } else {
+    static_assert(sizeof(T) == 4, "a 16-bit gradient accompanies float data only");
+    const uint16_t *h = (const uint16_t *)dy + e;
+    if constexpr (VEC == 4) {
+      const u32x2 v = *(const u32x2 *)h;
+      const uint32_t lo = v.x, hi = v.y;
+      return f32x4{__builtin_bit_cast(float, lo), __builtin_bit_cast(float, hi), 0.f, 0.f};
+    } else {
+      return __builtin_bit_cast(float, (uint32_t)*h);
+    }
+  }
+}
+__device__ __forceinline__ float widen_16(uint32_t bits16, int dydtype) {
+  const float b = bf16_bits_to_float(bits16 << 16);
+  const float h = (float)__builtin_bit_cast(_Float16, (uint16_t)bits16);
+  return dydtype == GN_BF16 ? b : h;
+}
+template <typename T, int VEC, bool DY16>
+__device__ __forceinline__ void unpack_dy(typename LaneVec<T, VEC>::raw_t raw, acc_t<T> (&v)[VEC], int dydtype) {
+  if constexpr (!DY16) {
+    LaneVec<T, VEC>::unpack(raw, v);
+  } else if constexpr (VEC == 4) {
+    const float r0 = raw.x, r1 = raw.y;
+    const uint32_t lo = __builtin_bit_cast(uint32_t, r0), hi = __builtin_bit_cast(uint32_t, r1);
+    v[0] = widen_16(lo & 0xffffu, dydtype);
+    v[1] = widen_16(lo >> 16, dydtype);
+    v[2] = widen_16(hi & 0xffffu, dydtype);
+    v[3] = widen_16(hi >> 16, dydtype);
+  } else {
+    v[0] = widen_16(__builtin_bit_cast(uint32_t, raw) & 0xffffu, dydtype);
+  }
+}
+// One element of it (recovery paths, scalar code).
+template <typename T, bool DY16> __device__ __forceinline__ float load_dy_scalar(const T *dy, int64_t e, int dydtype) {
+  float v[1];
+  unpack_dy<T, 1, DY16>(load_dy<T, 1, DY16>(dy, e), v, dydtype);
+  return v[0];
+}
+
 // Per-group tile partials are stored as planes of one field each, laid out [N][nchunk][G][tiles]: the
 // entries a consumer merges for one group (all tiles of the one or two chunks that hold the group) are
 // contiguous, so the merge reads them with coalesced loads.
@@ -804,10 +850,10 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
 // gn_kernel.cu:786-797).
 //   partC : [N][tiles][C][2]      partG : 2 planes [N][nchunk][G][tiles]
 // ---------------------------------------------------------------------------------------------
-template <typename T, typename PT, int VEC, int ACT>
+template <typename T, typename PT, int VEC, int ACT, bool DY16 = false>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) void bwd_reduce_kernel(
     const T *__restrict__ x, const T *__restrict__ dy, const void *mean, const void *rstd, int sdtype, const void *w,
-    const void *b, acc_t<T> *__restrict__ partC, acc_t<T> *__restrict__ partG, Plan p) {
+    const void *b, acc_t<T> *__restrict__ partC, acc_t<T> *__restrict__ partG, Plan p, int dydtype) {
   using A = acc_t<T>;
   using LV = LaneVec<T, VEC>;
   constexpr int U = kUnrollBwd;
@@ -830,8 +876,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int64_t o = off + (int64_t)clamp_row(bi * U + u, sfl.rows) * step;
-        if constexpr (decltype(sel)::value == 0) { bx0[u] = LV::load(x + o); bd0[u] = LV::load(dy + o); }
-        else { bx1[u] = LV::load(x + o); bd1[u] = LV::load(dy + o); }
+        if constexpr (decltype(sel)::value == 0) { bx0[u] = LV::load(x + o); bd0[u] = load_dy<T, VEC, DY16>(dy, o); }
+        else { bx1[u] = LV::load(x + o); bd1[u] = load_dy<T, VEC, DY16>(dy, o); }
       }
     };
     auto consume = [&](auto sel, int bi) {
@@ -839,8 +885,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
       for (int u = 0; u < U; ++u) {
         const A keep = bi * U + u < rows ? (A)1 : (A)0;
         A vx[VEC], vd[VEC];
-        if constexpr (decltype(sel)::value == 0) { LV::unpack(bx0[u], vx); LV::unpack(bd0[u], vd); }
-        else { LV::unpack(bx1[u], vx); LV::unpack(bd1[u], vd); }
+        if constexpr (decltype(sel)::value == 0) { LV::unpack(bx0[u], vx); unpack_dy<T, VEC, DY16>(bd0[u], vd, dydtype); }
+        else { LV::unpack(bx1[u], vx); unpack_dy<T, VEC, DY16>(bd1[u], vd, dydtype); }
 #pragma unroll
         for (int j = 0; j < VEC; ++j) {
           const A g = keep * vd[j] * act_bwd<ACT, A>(vx[j] * sa[j] + sb[j]);
@@ -1012,11 +1058,11 @@ __global__ __launch_bounds__(kBlock) void bwd_compact_kernel(const A *__restrict
 // One extra column of workgroups (blockIdx.x == tiles, sample 0 only) produces, for the channels of its
 // chunk, dgamma_c = sum_n (S1 - mean S2) rstd and dbeta_c = sum_n S2 (compute_dweight_dbias, gn_kernel.cu:695-728).
 // ---------------------------------------------------------------------------------------------
-template <typename T, typename PT, int VEC, int ACT>
+template <typename T, typename PT, int VEC, int ACT, bool DY16 = false>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) void bwd_dx_kernel(
     const T *__restrict__ x, const T *__restrict__ dy, T *__restrict__ dx, const void *mean, const void *rstd, int sdtype,
     const void *w, const void *b, const acc_t<T> *__restrict__ partC, const acc_t<T> *__restrict__ partG, PartialGeo q,
-    void *dw, void *db, Plan p) {
+    void *dw, void *db, Plan p, int dydtype) {
   using A = acc_t<T>;
   using LV = LaneVec<T, VEC>;
   constexpr int U = kUnrollBwd;
@@ -1078,16 +1124,16 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int64_t o = off + (int64_t)clamp_row(bi * U + u, sfl.rows) * step;
-        if constexpr (decltype(sel)::value == 0) { bx0[u] = LV::load(x + o); bd0[u] = LV::load(dy + o); }
-        else { bx1[u] = LV::load(x + o); bd1[u] = LV::load(dy + o); }
+        if constexpr (decltype(sel)::value == 0) { bx0[u] = LV::load(x + o); bd0[u] = load_dy<T, VEC, DY16>(dy, o); }
+        else { bx1[u] = LV::load(x + o); bd1[u] = load_dy<T, VEC, DY16>(dy, o); }
       }
     };
     auto consume = [&](auto sel, int bi) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         A vx[VEC], vd[VEC];
-        if constexpr (decltype(sel)::value == 0) { LV::unpack(bx0[u], vx); LV::unpack(bd0[u], vd); }
-        else { LV::unpack(bx1[u], vx); LV::unpack(bd1[u], vd); }
+        if constexpr (decltype(sel)::value == 0) { LV::unpack(bx0[u], vx); unpack_dy<T, VEC, DY16>(bd0[u], vd, dydtype); }
+        else { LV::unpack(bx1[u], vx); unpack_dy<T, VEC, DY16>(bd1[u], vd, dydtype); }
 #pragma unroll
         for (int j = 0; j < VEC; ++j) {
           const A g = vd[j] * act_bwd<ACT, A>(vx[j] * sa[j] + sb[j]);

@@ -29,6 +29,7 @@ SYMBOLS = (
     "gnnhwc_fwd_static",
     "gnnhwc_fwd_static_scratch_bytes",
     "gnnhwc_bwd",
+    "gnnhwc_bwd_cast",
     "gnnhwc_nchw_workspace_bytes",
     "gnnhwc_fwd_nchw",
     "gnnhwc_bwd_nchw",
@@ -72,6 +73,8 @@ def _load():
     lib.gnnhwc_fwd_static_scratch_bytes.restype = sz
     lib.gnnhwc_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, ci, ci, ci, ci, vp, sz, vp]
     lib.gnnhwc_bwd.restype = ci
+    lib.gnnhwc_bwd_cast.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, ci, ci, ci, ci, ci, vp, sz, vp]
+    lib.gnnhwc_bwd_cast.restype = ci
     lib.gnnhwc_nchw_workspace_bytes.argtypes = [i64, i64, i64, i64, ci, ci]
     lib.gnnhwc_nchw_workspace_bytes.restype = sz
     lib.gnnhwc_fwd_nchw.argtypes = list(lib.gnnhwc_fwd.argtypes)

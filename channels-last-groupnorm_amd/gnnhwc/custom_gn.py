@@ -190,8 +190,10 @@ def gn_nhwc_bwd(dy, X, weight, bias, means, rstds, G, act_fn_option):
     dt = _dtype_code(X, "X")
     pdt, w_ptr, b_ptr, _keep = _param_args(weight, bias, C, dt)
     sdt = _dtype_code(means, "means")
-    if dy.dtype != X.dtype:
-        raise RuntimeError("dy and X must have the same dtype (%s vs %s)" % (dy.dtype, X.dtype))
+    # (float data may come with a 16-bit gradient: the backward of gnop::fwd_cast; the kernels widen it as they load it)
+    dy16 = X.dtype == torch.float32 and dy.dtype in (torch.float16, torch.bfloat16)
+    if dy.dtype != X.dtype and not dy16:
+        raise RuntimeError("dy and X must have the same dtype, or dy float16 / bfloat16 with float32 X (%s vs %s)" % (dy.dtype, X.dtype))
     if rstds.dtype != means.dtype:
         raise RuntimeError("means and rstds must share a dtype")
     if means.numel() != N * G or rstds.numel() != N * G:
@@ -209,11 +211,11 @@ def gn_nhwc_bwd(dy, X, weight, bias, means, rstds, G, act_fn_option):
             raise RuntimeError("gnop::bwd: " + _cabi.last_error())
         stream = _current_stream_ptr(X.device)
         ws = _workspace(nbytes, X.device, stream)
-        rc = lib.gnnhwc_bwd(
+        rc = lib.gnnhwc_bwd_cast(
             dy_nrc.data_ptr(), X_nrc.data_ptr(), w_ptr, b_ptr,
             means.contiguous().data_ptr(), rstds.contiguous().data_ptr(),
             dX.data_ptr(), dweight.data_ptr() if dweight is not None else None, dbias.data_ptr() if dbias is not None else None,
-            N, R, C, G, int(act_fn_option), dt, pdt, sdt,
+            N, R, C, G, int(act_fn_option), dt, pdt, sdt, _dtype_code(dy, "dy"),
             ws.data_ptr(), ws.numel(), stream)
     _cabi.check(rc, "gnop::bwd")
     return dX.permute(0, 2, 1), dweight, dbias
@@ -260,8 +262,10 @@ def gn_nchw_bwd(dy, X, weight, bias, means, rstds, G, act_fn_option):
     dt = _dtype_code(X, "X")
     pdt, w_ptr, b_ptr, _keep = _param_args(weight, bias, C, dt)
     sdt = _dtype_code(means, "means")
-    if dy.dtype != X.dtype:
-        raise RuntimeError("dy and X must have the same dtype (%s vs %s)" % (dy.dtype, X.dtype))
+    # (float data may come with a 16-bit gradient: the backward of gnop::fwd_cast; the kernels widen it as they load it)
+    dy16 = X.dtype == torch.float32 and dy.dtype in (torch.float16, torch.bfloat16)
+    if dy.dtype != X.dtype and not dy16:
+        raise RuntimeError("dy and X must have the same dtype, or dy float16 / bfloat16 with float32 X (%s vs %s)" % (dy.dtype, X.dtype))
     if rstds.dtype != means.dtype:
         raise RuntimeError("means and rstds must share a dtype")
     if means.numel() != N * G or rstds.numel() != N * G:
@@ -451,9 +455,9 @@ def _fwd_cast_setup_context(ctx, inputs, output):
 
 
 def _fwd_cast_backward(ctx, dY, _dmeans, _drstds):
-    """The backward kernels have one element type: the 16-bit gradient of Y is widened to X's float32 first."""
+    """The 16-bit gradient of Y goes to the backward kernels as it is (gnnhwc_bwd_cast widens it in registers)."""
     X, weight, bias, means, rstds = ctx.saved_tensors
-    dY = dY.permute(0, 2, 1).to(X.dtype).contiguous().permute(0, 2, 1)
+    dY = dY.permute(0, 2, 1).contiguous().permute(0, 2, 1)
     if weight is None:
         dX, _dw, _db = gn_nhwc_bwd(dY, X, None, None, means, rstds, ctx.G, ctx.act_fn_option)
         return dX, None, None, None, None, None, None

@@ -112,8 +112,7 @@ int gnnhwc_fwd(const void *x, const void *weight, const void *bias,
  *   y_dtype : GNNHWC_F16 or GNNHWC_BF16 (type of y); GNNHWC_F32 makes this gnnhwc_fwd.  Anything else, or another
  *             dtype with a y_dtype different from it, is GNNHWC_ERR_INVALID_ARGUMENT.
  * y must not be the buffer of x when the types differ.  Everything else as gnnhwc_fwd (same workspace size).
- * A backward that follows takes dy in dtype: gnnhwc_bwd has one element type, so a 16-bit incoming gradient is
- * widened by the caller first.
+ * The backward that follows is gnnhwc_bwd_cast, which reads the 16-bit gradient of y as it is.
  */
 int gnnhwc_fwd_cast(const void *x, const void *weight, const void *bias,
                     void *y, void *mean, void *rstd,
@@ -183,6 +182,23 @@ int gnnhwc_bwd(const void *dy, const void *x, const void *weight, const void *bi
                int64_t N, int64_t R, int64_t C, int64_t G, int act,
                int dtype, int param_dtype, int stats_dtype,
                void *workspace, size_t workspace_bytes, void *stream /* hipStream_t */);
+
+/*
+ * Backward of float data whose incoming gradient is stored in a 16-bit type (no counterpart in the reference, where dy
+ * has the type of x, custom_gn.cpp:64-65): the training half of gnnhwc_fwd_cast.  dy is widened in registers as it is
+ * loaded; no separate pass over it, and dy costs S/2 instead of S bytes of traffic.
+ *   dtype    : GNNHWC_F32 (type of x and dx).
+ *   dy_dtype : GNNHWC_F16 or GNNHWC_BF16 (type of dy); GNNHWC_F32 makes this gnnhwc_bwd.  Anything else, or another
+ *              dtype with a dy_dtype different from it, is GNNHWC_ERR_INVALID_ARGUMENT.
+ * dx must not be the buffer of dy when the types differ.  Results are bit for bit those of gnnhwc_bwd on dy widened to
+ * float.  Everything else as gnnhwc_bwd (same workspace size).
+ */
+int gnnhwc_bwd_cast(const void *dy, const void *x, const void *weight, const void *bias,
+                    const void *mean, const void *rstd,
+                    void *dx, void *dweight, void *dbias,
+                    int64_t N, int64_t R, int64_t C, int64_t G, int act,
+                    int dtype, int param_dtype, int stats_dtype, int dy_dtype,
+                    void *workspace, size_t workspace_bytes, void *stream /* hipStream_t */);
 
 /*
  * Channels-first layout: x, y, dy, dx are (N, C, R) contiguous, R fastest.  The reference has no kernel for it:

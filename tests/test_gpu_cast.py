@@ -1,4 +1,7 @@
-"""GPU parity of gnnhwc_fwd_cast: float32 data, y written as float16 / bfloat16 by the kernel.
+"""GPU parity of gnnhwc_fwd_cast and gnnhwc_bwd_cast: float32 data, y written / dy read as float16 / bfloat16 by the kernels.
+
+gnnhwc_bwd_cast: dx, dweight, dbias are bit for bit those of gnnhwc_bwd on the same gradient widened to float32 first (the
+kernels widen exactly, in registers), for both kernel families and the scalar kernels; errors as gnnhwc_fwd_cast's.
 
 Bars: y is bit for bit gnnhwc_fwd's float32 y rounded once (round to nearest even) to the 16-bit type -- the kernel
 rounds the very fp32 value the plain forward stores -- and therefore within one rounding of the float64 oracle's y
@@ -12,7 +15,7 @@ import torch
 
 from oracle import gn_oracle as orc
 from gnnhwc import _cabi
-from tests.gpu_harness import DT_CODE, _ptr, as_np64, cabi_fwd, err
+from tests.gpu_harness import DT_CODE, _ptr, as_np64, cabi_bwd, cabi_fwd, err
 
 pytestmark = pytest.mark.gpu
 
@@ -140,3 +143,60 @@ def test_cast_through_the_python_surface(affine, device):
     m2 = GN_NHWC(8, 64, activation="silu", out_dtype=torch.float32, affine=affine).to(device)
     assert m2(x.detach().bfloat16()).dtype == torch.float32
     assert m(x.detach().contiguous()).dtype == torch.bfloat16
+
+
+def cabi_bwd_cast(dy, x, w, b, mean, rstd, G, act, dx=None, dtype_code=None, dy_code=None):
+    N, R, C = x.shape
+    dt = DT_CODE[x.dtype] if dtype_code is None else dtype_code
+    dx = torch.empty_like(x) if dx is None else dx
+    dw = torch.empty((C,), dtype=w.dtype, device=x.device) if w is not None else None
+    db = torch.empty((C,), dtype=w.dtype, device=x.device) if w is not None else None
+    lib = _cabi.lib
+    nbytes = lib.gnnhwc_bwd_workspace_bytes(N, R, C, G, DT_CODE[x.dtype])
+    assert nbytes > 0, _cabi.last_error()
+    ws = torch.empty((nbytes,), dtype=torch.uint8, device=x.device)
+    rc = lib.gnnhwc_bwd_cast(_ptr(dy), _ptr(x), _ptr(w), _ptr(b), _ptr(mean), _ptr(rstd), _ptr(dx), _ptr(dw), _ptr(db), N, R, C, G,
+                             int(act), dt, DT_CODE[w.dtype] if w is not None else dt, DT_CODE[mean.dtype],
+                             DT_CODE[dy.dtype] if dy_code is None else dy_code, _ptr(ws), ws.numel(),
+                             ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    return rc, dx, dw, db
+
+
+@pytest.mark.parametrize("dy_dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape,G", SHAPES + [((5, 128 * 128, 320), 32)])  # the last: a backward in two launches
+def test_cast_backward_matches_widen_then_backward(family, shape, G, dy_dtype, device):
+    act_name = ACTS[(shape[1] + shape[2] + 1) % 5]
+    act = orc.ACT_CODES[act_name]
+    print("bwd_cast", family, shape, G, act_name, dy_dtype, flush=True)
+    x, w, b = _inputs(shape, device, 23)
+    gen = torch.Generator().manual_seed(29)
+    dy16 = torch.randn(shape, generator=gen).to(dy_dtype).to(device)
+    _y, mean, rstd = cabi_fwd(x, w, b, G, EPS, act)
+    want = cabi_bwd(dy16.float(), x, w, b, mean, rstd, G, act)  # today's sequence: widen, then the float backward
+    rc, dx, dw, db = cabi_bwd_cast(dy16, x, w, b, mean, rstd, G, act)
+    _cabi.check(rc, "gnnhwc_bwd_cast")
+    torch.cuda.synchronize()
+    for name, got, ref in (("dx", dx, want[0]), ("dweight", dw, want[1]), ("dbias", db, want[2])):
+        assert torch.equal(got, ref), "%s differs from the backward on the widened gradient" % name
+    # without parameters, and float32 dy through the same entry point (= gnnhwc_bwd)
+    rc, dx0, _, _ = cabi_bwd_cast(dy16, x, None, None, mean, rstd, G, act)
+    _cabi.check(rc, "gnnhwc_bwd_cast")
+    want0 = cabi_bwd(dy16.float(), x, None, None, mean, rstd, G, act, want_dw=False, want_db=False)
+    rc, dx1, dw1, db1 = cabi_bwd_cast(dy16.float(), x, w, b, mean, rstd, G, act)
+    _cabi.check(rc, "gnnhwc_bwd_cast")
+    torch.cuda.synchronize()
+    assert torch.equal(dx0, want0[0])
+    assert torch.equal(dx1, want[0]) and torch.equal(dw1, want[1]) and torch.equal(db1, want[2])
+
+
+def test_cast_backward_argument_errors(device):
+    x, w, b = _inputs((2, 64, 32), device, 3)
+    _y, mean, rstd = cabi_fwd(x, w, b, 4, EPS, 2)
+    dy = torch.randn_like(x).to(torch.bfloat16)
+    assert cabi_bwd_cast(dy, x, w, b, mean, rstd, 4, 2, dy_code=1)[0] == -1        # float64 gradient of float32 data
+    assert cabi_bwd_cast(dy, x, w, b, mean, rstd, 4, 2, dy_code=7)[0] == -1        # unknown code
+    xb = x.to(torch.bfloat16)
+    wb, bb = w.to(torch.bfloat16), b.to(torch.bfloat16)
+    assert cabi_bwd_cast(dy.to(torch.float16), xb, wb, bb, mean, rstd, 4, 2)[0] == -1  # 16-bit data take dy in their own type
+    assert cabi_bwd_cast(dy, xb, wb, bb, mean, rstd, 4, 2)[0] == 0
+    torch.cuda.synchronize()
