@@ -20,11 +20,12 @@
 //    A consumer that sees this call's epoch in a record takes the values it loaded with it.  The epoch is a fresh
 //    64-bit value per call, so the workspace never needs clearing, there are no flags, and one memory round trip
 //    carries both "ready" and the data.
-//    This relies on an aligned 128-bit device-scope store being observed as a whole by an aligned 128-bit
-//    device-scope load (single-copy atomicity of a 16-byte access inside one 64-byte sector of the memory channel
-//    that owns it).  The instruction set does not promise it in writing; if it did not hold, a consumer could pair a
-//    fresh epoch with stale values.  The epoch therefore sits in the LAST two words of the record: a torn access
-//    that delivered the words in address order would show stale epoch words, not stale values.
+//    An aligned 128-bit device-scope store is expected to be observed as a whole by an aligned 128-bit device-scope
+//    load (single-copy atomicity of a 16-byte access inside one 64-byte sector of the memory channel that owns it),
+//    but the instruction set does not promise that in writing, so the protocol does not depend on it: the record
+//    validates itself.  Its third word is the low half of the epoch folded with a hash of the two values (record_hash),
+//    its fourth the high half: whichever words of a torn access are the stale ones, the record fails validation and
+//    is polled again.
 // Polling is bounded (SyncArea::max_spins).  When a wait of any lane expires (the workgroup that owes it a record is
 // not resident yet: something else holds part of the device), the whole workgroup leaves the fast path at the next
 // barrier and finishes its tile the slow way (recover_* below): it takes the records that have arrived, RECOMPUTES the
@@ -116,18 +117,29 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t record_region(const SyncArea &
 __device__ __forceinline__ RecordArray record_buffer(const SyncArea &s) { return {record_region(s), (int)s.rec_first}; }
 __device__ __forceinline__ RecordArray channel_record_buffer(const SyncArea &s) { return {record_region(s), (int)s.crec_first}; }
 __device__ __forceinline__ RecordArray final_record_buffer(const SyncArea &s) { return {record_region(s), (int)s.frec_first}; }
+// The third word of a record carries the low half of the epoch folded with a hash of the two values: a record whose four
+// words were not written together (an access observed in pieces, should that ever happen) does not validate, whichever
+// of its words are the stale ones, and is simply polled again.
+__device__ __forceinline__ unsigned record_hash(unsigned u0, unsigned u1) { return u0 ^ __builtin_amdgcn_alignbit(u1, u1, 13); }
 __device__ __forceinline__ void record_store(const RecordArray &r, int64_t idx, float v0, float v1, unsigned long long epoch) {
-  const u32x4 rec = {__builtin_bit_cast(unsigned, v0), __builtin_bit_cast(unsigned, v1), (unsigned)epoch,
-                     (unsigned)(epoch >> 32)};
+  const unsigned u0 = __builtin_bit_cast(unsigned, v0), u1 = __builtin_bit_cast(unsigned, v1);
+  const u32x4 rec = {u0, u1, (unsigned)epoch ^ record_hash(u0, u1), (unsigned)(epoch >> 32)};
   __builtin_amdgcn_raw_buffer_store_b128(rec, r.rsrc, ((int)idx + r.first) * 16, 0, kAuxDeviceScope);
 }
 __device__ __forceinline__ u32x4 record_load(const RecordArray &r, int64_t idx) {
   return __builtin_amdgcn_raw_buffer_load_b128(r.rsrc, ((int)idx + r.first) * 16, 0, kAuxDeviceScope);
 }
 __device__ __forceinline__ bool record_ready(const u32x4 &rec, unsigned long long epoch) {
-  return rec.z == (unsigned)epoch && rec.w == (unsigned)(epoch >> 32);
+  return (rec.z ^ record_hash(rec.x, rec.y)) == (unsigned)epoch && rec.w == (unsigned)(epoch >> 32);
 }
 
+// Lanes per group for the exchange: a lane takes kRecFast records per round trip, so half as many lanes as a group has
+// records serve it in one round -- and twice as many groups of the chunk are merged side by side, which for chunks that
+// hold many small groups (64 channels of groups of 10) saves the second pass over the groups and its round trip.
+__device__ __forceinline__ int exchange_lanes(const PartialGeo &q, int D) {
+  const int records = q.tiles * (div_by(D - 1, q.by_chunk) + 2);
+  return pow2_ceil_clamped((records + kRecFast - 1) / kRecFast, 64);
+}
 // Elements behind record (tile t, chunk k, group g): the rows of the tile times the channels of g in chunk k.
 // (32-bit arithmetic: channel indices and the rows of a tile fit, and 64-bit multiplies are slow here)
 __device__ __forceinline__ float record_count(const Plan &p, int t, int k, int g) {
@@ -899,7 +911,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
   } else {
     // merge the records of the chunk's groups (exact two-pass form, compute_stats_pt2's job:
     // src/gnnhwc/csrc/gn_kernel.cu:226-292); rstd = 1 / sqrt(M2 / n + eps)
-    const int L = merge_lanes(q, p.D);
+    const int L = exchange_lanes(q, p.D);
     const int nseg = kBlock >> __builtin_ctz(L);  // L is a power of two
     const int seg = threadIdx.x >> __builtin_ctz(L), sl = threadIdx.x & (L - 1);
     const A total = (A)p.D * (A)p.R;  // elements of a group
@@ -1255,7 +1267,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
       sm2[gi] = k2;
     }
   } else {
-    const int L = merge_lanes(q, p.D);
+    const int L = exchange_lanes(q, p.D);
     const int nseg = kBlock >> __builtin_ctz(L);  // L is a power of two
     const int seg = threadIdx.x >> __builtin_ctz(L), sl = threadIdx.x & (L - 1);
     for (int base = 0; base < l.ng; base += nseg) {
