@@ -213,7 +213,10 @@ inline void launch(int kind, void (*kernel)(KArgs...), dim3 grid, dim3 block, hi
   hipEvent_t e0 = nullptr, e1 = nullptr;
   if ((kind == kKindFusedFwd || kind == kKindFusedBwd || kind == kKindFusedFwdAdd) && cooperative_launches()) {
     std::tuple<KArgs...> vals(static_cast<KArgs>(args)...);
+    const bool timed = profile_events(kind, &e0, &e1);  // (events around the launch, not bound to the dispatch)
+    if (timed) (void)hipEventRecord(e0, stream);
     launch_cooperative(kernel, grid, block, stream, vals, std::index_sequence_for<KArgs...>{});
+    if (timed) (void)hipEventRecord(e1, stream);
     return;
   }
   if (profile_events(kind, &e0, &e1))

@@ -102,3 +102,36 @@ def test_static_forward_rejects_what_its_scratch_cannot_hold(device):
     # invalid shapes are refused like everywhere else, and an empty batch is a no-op
     assert _cabi.lib.gnnhwc_fwd_static(None, None, None, None, None, None, 1, 16, 7, 3, EPS, 0, 0, 0, 0, None) == -1
     assert _cabi.lib.gnnhwc_fwd_static(None, None, None, None, None, None, 0, 16, 8, 2, EPS, 0, 0, 0, 0, None) == 0
+
+
+def test_static_forward_allocates_nothing_under_graph_capture(device):
+    """After one warm-up call per device (which looks up the scratch address), the call is recorded into a HIP graph with
+    the capture in 'global' error mode -- any allocation, event creation or host-pinned allocation the library made
+    while the stream is capturing would invalidate the capture -- and every replay reproduces the eager result bit for bit."""
+    shape, G, dtype, act = (2, 4096, 320), 32, torch.bfloat16, orc.ACT_CODES["silu"]
+    x, w, b = _inputs(shape, dtype, device, 7)
+    rc, y_eager, mean_eager, rstd_eager = fwd_static(x, w, b, G, act)  # warm-up: the only call that may touch set-up paths
+    _cabi.check(rc, "gnnhwc_fwd_static")
+    torch.cuda.synchronize()
+    N, R, C = shape
+    y = torch.empty_like(x)
+    mean = torch.empty((N, G), dtype=torch.float32, device=device)
+    rstd = torch.empty((N, G), dtype=torch.float32, device=device)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side, capture_error_mode="global"):
+            rc = _cabi.lib.gnnhwc_fwd_static(_ptr(x), _ptr(w), _ptr(b), _ptr(y), _ptr(mean), _ptr(rstd), N, R, C, G, EPS, int(act),
+                                             DT_CODE[dtype], DT_CODE[dtype], 0, ctypes.c_void_p(side.cuda_stream))
+    _cabi.check(rc, "gnnhwc_fwd_static under capture")
+    torch.cuda.current_stream().wait_stream(side)
+    for replay in range(3):
+        y.zero_()
+        mean.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, y_eager) and torch.equal(mean, mean_eager) and torch.equal(rstd, rstd_eager), "replay %d" % replay
+        _ = fwd_static(x, w, b, G, act)  # eager work of the same kind between the replays
+        torch.cuda.synchronize()
