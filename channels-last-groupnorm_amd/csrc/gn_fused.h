@@ -694,8 +694,10 @@ __device__ __forceinline__ void recover_bwd_tail(const T *x, const T *dy, int dy
 //   records : {mean, M2, epoch} per (n, chunk, group, tile)
 // ---------------------------------------------------------------------------------------------
 // Occupancy the register budget is sized for.
+// (with a residual: the tile plus a window of residual_window(nv) rows of the residual)
+constexpr int residual_window(int nv) { return nv <= 8 ? nv : 8; }
 constexpr int fused_fwd_waves(int nv, int add) {
-  return add == kAddResidual ? (nv <= 4 ? 4 : nv <= 8 ? 3 : nv <= 16 ? 2 : 1) : (nv <= 8 ? 4 : nv <= 16 ? 3 : 2);
+  return add == kAddResidual ? (nv <= 4 ? 4 : nv <= 16 ? 3 : 2) : (nv <= 8 ? 4 : nv <= 16 ? 3 : 2);
 }
 // TWO_LEVEL: the exchange of a launch with many row tiles per sample (two_level_exchange on the host).  A template
 // parameter, not a run-time switch: the code of the form a launch does not use would sit in the middle of the path every
@@ -763,25 +765,31 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_fw
     if constexpr (ADD == kAddResidual) {
       // (an absent residual would re-read x and be discarded, so that the loads stay free of branches; the host
       // picks the channel-only variant for that case)
+      // The residual passes through a window of RW rows: row u + RW is requested into the slot of row u as soon as that
+      // row has been added, so the kernel holds NV + RW rows at most, not 2 NV -- which is what lets a tensor of the
+      // size of the plain forward's (x alone fills the registers) still run as one launch with its residual.
+      constexpr int RW = residual_window(NV);
       const T *rp = add.residual ? (const T *)add.residual : x;
       const bool has_r = add.residual != nullptr;
-      typename LV::raw_t rbuf[NV];
+      typename LV::raw_t rbuf[RW];
 #pragma unroll
-      for (int u = 0; u < NV; ++u) {
-        const int64_t o = off + (int64_t)clamp_row(u, rows) * step;
-        buf[u] = LV::load(x + o);
-        rbuf[u] = LV::load(rp + o);
-      }
+      for (int u = 0; u < RW; ++u) rbuf[u] = LV::load(rp + off + (int64_t)clamp_row(u, rows) * step);
+#pragma unroll
+      for (int u = 0; u < NV; ++u) buf[u] = LV::load(x + off + (int64_t)clamp_row(u, rows) * step);
       T *so = sum_after_exchange<T>(x, add) ? nullptr : (T *)add.sum_out;
 #pragma unroll
       for (int u = 0; u < NV; ++u) {
         A vx[VEC], vr[VEC];
         LV::unpack(buf[u], vx);
-        LV::unpack(rbuf[u], vr);
+        LV::unpack(rbuf[u % RW], vr);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) vx[j] = (vx[j] + (has_r ? vr[j] : (A)0)) + tb[j];
         buf[u] = LV::pack(vx);  // rounded to T once: the statistics and y are those of the stored sum
         if (so && u < rows) store_streaming<LV>(so + off + (int64_t)u * step, buf[u]);
+        if (u + RW < NV) {
+          issue_order_fence();  // not before the row it replaces has been used: the slot is the register budget
+          rbuf[u % RW] = LV::load(rp + off + (int64_t)clamp_row(u + RW, rows) * step);
+        }
       }
     } else {
 #pragma unroll
