@@ -68,6 +68,12 @@ def parse_args():
     ap.add_argument("--switch-cost", action="store_true",
                     help="no headline: event-timed duration of each kernel of the workload when it follows itself and when it "
                          "follows a different kernel whose data is tiny (a 1 MB plain copy; a small GroupNorm forward)")
+    ap.add_argument("--recovery-cost", action="store_true",
+                    help="no headline: event-timed duration of each kernel of the workload on the fast path and with every wait "
+                         "forced to expire (every workgroup recomputes the records it needs): the worst case of the recovery path")
+    ap.add_argument("--load-ceiling", action="store_true",
+                    help="no headline: the load phase of each single-launch kernel of the workload on its own (a kernel that only "
+                         "requests the rows), beside the kernel itself, on cold tensors")
     ap.add_argument("--code-placement", action="store_true",
                     help="no headline: per-kernel times of the workload (event-timed inside the sweep) in four child processes that "
                          "first load 0, 1, 2, 3 copies of the library under other names, which moves the code of the library proper "
@@ -599,6 +605,106 @@ def switch_cost(names, device):
         torch.cuda.empty_cache()
 
 
+def recovery_cost(names, device):
+    """What the recovery path of the single-launch kernels costs in the worst case: every wait of every workgroup is made to
+    expire at its first poll (poll limit -2), so every workgroup recomputes every record it needs from the inputs and reads
+    its rows again.  Event-timed microseconds per launch, next to the same launch on the fast path."""
+    import torch
+    from gnnhwc import _cabi
+    import workloads as configs
+
+    stream = torch.cuda.current_stream().cuda_stream
+    lib = _cabi.lib
+    print("# event-timed microseconds per launch: fast path | every workgroup on the recovery path (poll limit -2)")
+    print("%-6s %-4s %12s %14s %8s" % ("shape", "pass", "fast path", "all recover", "x"))
+    for name in names:
+        p = Problem(configs.CONFIGS[name], device)
+        for which in (("fwd", "bwd") if p.bwd else ("fwd",)):
+            row = []
+            for limit in (-1, -2):
+                prev = lib.gnnhwc_debug_set_spin_limit(limit)
+                try:
+                    for _ in range(5):
+                        p.step(0, stream, which)
+                    torch.cuda.synchronize()
+                    _cabi.profile_collect()
+                    _cabi.profile_enable(True)
+                    for _ in range(20):
+                        p.step(0, stream, which)
+                    _cabi.profile_enable(False)
+                    torch.cuda.synchronize()
+                    res = {k: ms / n * 1e3 for k, (n, ms) in _cabi.profile_collect().items() if n}
+                    row.append(sum(res.values()))
+                finally:
+                    lib.gnnhwc_debug_set_spin_limit(prev)
+            lib.gnnhwc_resident_status()
+            print("%-6s %-4s %12.2f %14.1f %8.0f" % (name, which, row[0], row[1], row[1] / row[0]))
+        del p
+        torch.cuda.empty_cache()
+
+
+def load_ceiling(names, device):
+    """The load phase of the single-launch kernels on its own: a kernel with their grid and tile geometry whose lanes request
+    all their rows up front and do nothing else (gnnhwc_debug_load_tile), on cold tensors (eight sets in rotation).  No
+    single-launch kernel can have its rows sooner; next to it the library's kernels on the same rotation of cold tensors."""
+    import re
+    import torch
+    from gnnhwc import _cabi
+    import workloads as configs
+
+    stream = torch.cuda.current_stream().cuda_stream
+    lib = _cabi.lib
+    print("# event-timed microseconds per launch on cold tensors (8 sets of buffers in rotation)")
+    print("%-6s %-4s %-44s %10s %10s %12s" % ("shape", "pass", "kernel", "kernel us", "loads us", "loads GB/s"))
+    for name in names:
+        cfg = configs.CONFIGS[name]
+        p = Problem(cfg, device, 8)
+        row_bytes = p.C * (p.S // (p.N * p.R * p.C))
+        for which in (("fwd", "bwd") if p.bwd else ("fwd",)):
+            p.step(0, stream, which)
+            inst = _cabi.last_launch()
+            m = re.search(r"rows=(\d+)", inst)
+            ctr = [0]
+
+            def kernel():
+                p.step(ctr[0] % 8, stream, which)
+                ctr[0] += 1
+
+            def loads():
+                b = p.sets[ctr[0] % 8]
+                ctr[0] += 1
+                _cabi.check(lib.gnnhwc_debug_load_tile(b["x"].data_ptr(), b["dy"].data_ptr() if which == "bwd" else None, None, p.N, p.R,
+                                                       row_bytes, int(m.group(1)), stream), "gnnhwc_debug_load_tile")
+
+            row = []
+            for fn in (kernel, loads):
+                if fn is loads and (m is None or row_bytes % 128 != 0):
+                    row.append(float("nan"))
+                    continue
+                blocks = []
+                for _ in range(2):  # the smaller of two blocks of 48 launches (the first block after a reallocation can run slow)
+                    for _ in range(16):
+                        fn()
+                    torch.cuda.synchronize()
+                    _cabi.profile_collect()
+                    _cabi.profile_enable(True)
+                    for _ in range(48):
+                        fn()
+                    _cabi.profile_enable(False)
+                    torch.cuda.synchronize()
+                    res = {k: ms / n * 1e3 for k, (n, ms) in _cabi.profile_collect().items() if n}
+                    blocks.append(sum(res.values()))
+                row.append(min(blocks))
+                if max(blocks) > 2 * min(blocks):
+                    print("# %s %s %s: blocks of %.1f and %.1f us per launch" % (name, which, fn.__name__, blocks[0], blocks[1]))
+                if lib.gnnhwc_resident_status() != 0:
+                    raise RuntimeError("a single-launch kernel recomputed records during the probe: its time is not a load ceiling comparison")
+            nbytes = (2 if which == "bwd" else 1) * p.S
+            print("%-6s %-4s %-44s %10.2f %10.2f %12.0f" % (name, which, inst.replace(" ", ","), row[0], row[1], nbytes / (row[1] * 1e-6) / 1e9))
+        del p
+        torch.cuda.empty_cache()
+
+
 def code_placement_child(names, device, copies):
     """One process of --code-placement: load `copies` copies of the library first (each one's first kernel launch makes the
     runtime load a code object, which takes the next 2 MB-aligned slot), then time the workload's kernels inside the sweep."""
@@ -1090,6 +1196,12 @@ def main():
         return
     if args.results_table:
         results_table(args, device)
+        return
+    if args.load_ceiling:
+        load_ceiling(list(configs.SD_UNET_SWEEP) + ["c4a", "c4b", "c5b_bf16_silu"] if args.workload == "sd_unet" else [args.workload], device)
+        return
+    if args.recovery_cost:
+        recovery_cost(list(configs.SD_UNET_SWEEP) + ["c4a", "c2"] if args.workload == "sd_unet" else [args.workload], device)
         return
     if args.switch_cost:
         switch_cost(list(configs.SD_UNET_SWEEP) if args.workload == "sd_unet" else

@@ -41,6 +41,7 @@ SYMBOLS = (
     "gnnhwc_debug_read_trace",
     "gnnhwc_debug_plan",
     "gnnhwc_debug_last_launch",
+    "gnnhwc_debug_load_tile",
 )
 
 
@@ -93,6 +94,8 @@ def _load():
     lib.gnnhwc_debug_read_trace.restype = ci
     lib.gnnhwc_debug_set_spin_limit.argtypes = [ci]
     lib.gnnhwc_debug_set_spin_limit.restype = ci
+    lib.gnnhwc_debug_load_tile.argtypes = [vp, vp, vp, i64, i64, i64, ci, vp]
+    lib.gnnhwc_debug_load_tile.restype = ci
     lib.gnnhwc_debug_copy.argtypes = [vp, vp, sz, vp]
     lib.gnnhwc_debug_copy.restype = ci
     lib.gnnhwc_debug_plan.argtypes = [i64, i64, i64, i64, ci, ci, ci, ctypes.POINTER(i64)]

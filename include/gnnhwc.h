@@ -297,6 +297,16 @@ int gnnhwc_debug_last_launch(int64_t *out /* [7] */);
 int gnnhwc_debug_copy(void *dst, const void *src, size_t bytes, void *stream /* hipStream_t */);
 
 /*
+ * The load phase of a single-launch kernel on its own (no counterpart in the reference): every lane of a grid of
+ * (row tiles, 128-byte chunks, samples) workgroups requests rows_per_lane (4, 8, 16, 22 or 32) rows of 16 bytes of x --
+ * and of dy unless it is NULL -- up front, in those kernels' tile geometry, and nothing else happens.  A yardstick like
+ * gnnhwc_debug_copy: a single-launch kernel cannot have its rows sooner than this kernel ends.  row_bytes: bytes of one
+ * row of the (N, R, C) tensor, a multiple of 128.  sink: 4 writable bytes or NULL.  Timed as kernel kind 8.
+ */
+int gnnhwc_debug_load_tile(const void *x, const void *dy, void *sink, int64_t N, int64_t R, int64_t row_bytes,
+                           int rows_per_lane, void *stream /* hipStream_t */);
+
+/*
  * The tiling the multi-launch kernels would use for a problem (no counterpart in the reference, whose
  * calc_block_params, gn_kernel.cu:37-60, is internal too); nothing is launched, no GPU is needed.  For tests of the
  * host-side planning.  vector: 1 = 16-byte lane vectors (C must be a multiple of 16 / sizeof(dtype)), 0 = scalar
