@@ -1124,7 +1124,7 @@ def results_table(args, device):
     print("  copy kernel reading and writing one tensor of the same size (2 S); cpu us = torch.nn.functional.group_norm + activation (+ autograd)")
     print("  on %d host threads, same tensors; err = max |ours - truth| / (|truth| + rms(truth)) against the float64 oracle, observed / bar" % cpu["cores"])
     print("  (float32: bar 1e-5 and also the pure relative error over |truth| >= rms, in brackets; 16-bit: bar = torch's own error in that type + 2 %).")
-    print("  kernel = what the library launched (rows per lane of the register tile, x window rows, two-level exchange, launches per call).")
+    print("  kernel = what the library launched (rows per lane of the register tile, x window rows, rows of x parked in LDS, two-level exchange, launches per call).")
     print()
     hdr = "%-20s %-5s %-22s %7s %7s %8s %7s %6s | %7s %6s %7s %6s | %7s %9s | %-34s | %s" % (
         "config", "dtype", "shape (N,C,spatial) G", "fwd us", "bwd us", "f+b us", "GB/s", "%peak", "fwd MB", "ratio", "bwd MB", "ratio",
