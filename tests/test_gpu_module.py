@@ -501,6 +501,63 @@ def test_single_launch_kernels_recover_from_expired_waits(N, R, C, G, act, dtype
         _cabi.set_resident(before)
 
 
+@pytest.mark.parametrize("in_place", [False, True])
+@pytest.mark.parametrize("polls", [0, 2, 16])
+@pytest.mark.parametrize("N,R,C,G,act,dtype", RECOVERY_SHAPES)
+def test_short_waits_mix_arrived_and_recomputed_records(N, R, C, G, act, dtype, polls, in_place, device):
+    """The recovery as it happens in the field: with a poll limit of 0, 2 or 16 (not the forced mode) a wait expires
+    only when its record really has not arrived yet, so a launch is a mixture of workgroups on the fast path and
+    workgroups that take the records that have arrived and recompute the others.  The results must be those of an
+    undisturbed launch up to the rounding of a statistic (a recomputed record sums in another order) -- also when the
+    outputs replace the inputs in place (y in x's buffer, dx in dy's), where a recomputed record may only be used if its
+    owner has provably not stored anything yet."""
+    lib = _cabi.lib
+    gen = torch.Generator().manual_seed(77 + R + polls)
+    x = (torch.randn((N, R, C), generator=gen) * 2 + torch.randn((C,), generator=gen)).to(dtype).to(device)
+    dy = torch.randn((N, R, C), generator=gen).to(dtype).to(device)
+    w = (torch.rand(C, generator=gen) + 0.5).to(dtype).to(device)
+    b = (0.1 * torch.randn(C, generator=gen)).to(dtype).to(device)
+    code = orc.ACT_CODES[act]
+    half = dtype != torch.float32
+    before = _cabi.set_resident(True)
+    try:
+        y0, mean0, rstd0 = cabi_fwd(x, w, b, G, 1e-5, code)
+        dx0, dw0, db0 = cabi_bwd(dy, x, w, b, mean0, rstd0, G, code)
+        torch.cuda.synchronize()
+        prev = lib.gnnhwc_debug_set_spin_limit(polls)
+        recovered = 0
+        try:
+            lib.gnnhwc_resident_status()
+            for rep in range(3):
+                xin = x.clone() if in_place else x
+                dyin = dy.clone() if in_place else dy
+                _cabi.profile_collect()
+                _cabi.profile_enable(True)
+                y, mean, rstd = cabi_fwd(xin, w, b, G, 1e-5, code, y=xin if in_place else None)
+                dx, dw, db = cabi_bwd(dyin, x, w, b, mean0, rstd0, G, code, dx=dyin if in_place else None)
+                torch.cuda.synchronize()
+                _cabi.profile_enable(False)
+                launches = {k: v[0] for k, v in _cabi.profile_collect().items() if v[0]}
+                assert set(launches) == {"fused_fwd", "fused_bwd"}, launches
+                recovered += lib.gnnhwc_resident_status()
+                assert err(mean, mean0) <= 1e-5 and err(rstd, rstd0) <= 1e-5, (rep, "statistics")
+                # elementwise outputs: a statistic that differs in its last bits moves few elements by one spacing of the type
+                for name, a, t in (("y", y, y0), ("dx", dx, dx0)):
+                    assert err(a, t) <= (2.0 ** -7 if half else 1e-5), (rep, name, err(a, t))
+                    if half:
+                        assert float((a.float() != t.float()).float().mean()) < 0.02, (rep, name)
+                for name, a, t in (("dw", dw, dw0), ("db", db, db0)):
+                    assert err(a, t) <= (2.0 ** -7 if half else 1e-5), (rep, name, err(a, t))
+        finally:
+            _cabi.profile_enable(False)
+            lib.gnnhwc_debug_set_spin_limit(prev)
+        if polls == 0:
+            assert recovered > 0, "no wait expired although nobody waited at all"
+    finally:
+        lib.gnnhwc_resident_status()
+        _cabi.set_resident(before)
+
+
 def test_fused_additions_recover_from_expired_waits(device):
     """The same for the forward with fused additions (residual, per-sample channel addend, sum written out): the
     recomputation rebuilds the sum exactly as the fast path forms it."""
