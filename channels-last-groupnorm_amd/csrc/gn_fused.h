@@ -702,6 +702,20 @@ constexpr int fused_fwd_waves(int nv, int add) {
 // TWO_LEVEL: the exchange of a launch with many row tiles per sample (two_level_exchange on the host).  A template
 // parameter, not a run-time switch: the code of the form a launch does not use would sit in the middle of the path every
 // workgroup executes once, and these kernels are sensitive to their own size.
+
+// Rows of a backward tile that a lane requests before it starts on the first one; row u + upfront_rows follows when
+// row u has been consumed.  A CU serves the requests of its workgroups first come, first served: with every row
+// requested up front, the workgroup that came second gets its first row when the first one has its last, and then has
+// the arithmetic of its whole tile (15 operations and two transcendentals per element) ahead of it with nothing left to
+// overlap it.  Requested a few rows at a time, the requests of the workgroups of a CU interleave and all of them work
+// through their rows while rows are still arriving.  Four rows of x and of dy in flight per lane are what keeps the
+// memory system as busy as the whole tile did (measured: 3, 5, 6, 8 and 11 are all slower); the form that streams x
+// through a window keeps six of each.  The forward is left alone: it has a quarter of the arithmetic per row, and with
+// fewer rows in flight its rows only arrive later (c3c: 18.7 -> 21.7 us with 8 of 16 rows up front, 29 us with 4).
+constexpr int kUpfrontRows = 4;
+constexpr int kUpfrontWindowRows = 6;
+constexpr int upfront_rows(int nv) { return nv > kUpfrontRows ? kUpfrontRows : nv; }
+
 // The single parameter of the forward kernel (one block, so that the recovery path can read it again: reread_kernel_args).
 struct FusedFwdParams {
   const void *x;
@@ -1112,9 +1126,13 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
     gamma0 = w ? gv : (A)1;
   }
   issue_order_fence();
+  // NB rows of x and dy are requested up front, row u + NB as soon as row u has been consumed (see upfront_rows)
+  constexpr int NB = XW == 0 ? upfront_rows(NV) : NV;
+  constexpr int NBW = XW > 0 ? (kUpfrontWindowRows < NV ? kUpfrontWindowRows : NV) : NV;  // the same for dy beside a window of x
+  constexpr int NBX = XW > 0 ? (kUpfrontWindowRows < XW ? kUpfrontWindowRows : XW) : 0;    // and for the window itself
   if constexpr (XW == 0) {
 #pragma unroll
-    for (int u = 0; u < NV; ++u) {
+    for (int u = 0; u < NB; ++u) {
       const int64_t o = row_offset(u);
       bx[u] = LV::load(x + o);
       bd[u] = load_dy<T, VEC, DY16>(dy, o);
@@ -1123,9 +1141,9 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
     // the window of x first (row 0's arithmetic needs it), then all of dy; the rest of x follows row by row below
     const RowTerms t0 = fresh_terms();
 #pragma unroll
-    for (int u = 0; u < XW; ++u) bx[u] = LV::load(tile_row(x, t0, u));
+    for (int u = 0; u < NBX; ++u) bx[u] = LV::load(tile_row(x, t0, u));
 #pragma unroll
-    for (int u = 0; u < NV; ++u) bd[u] = load_dy<T, VEC, DY16>(dy_row(t0, u), 0);
+    for (int u = 0; u < NBW; ++u) bd[u] = load_dy<T, VEC, DY16>(dy_row(t0, u), 0);
   }
   commit_chunk_stats<A>(st, l, sm_mu, sm_rs);
   __builtin_amdgcn_s_setprio(2);  // towards the exchange: ahead of wavefronts that are already past theirs
@@ -1144,13 +1162,17 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
       if (rows != NV) {
         const typename LV::raw_t zero = {};
 #pragma unroll
-        for (int u = 0; u < NV; ++u)
+        for (int u = 0; u < (XW > 0 ? NBW : NB); ++u)
           if (u >= rows) bd[u] = zero;
       }
       const RowTerms t1 = fresh_terms();
 #pragma unroll
       for (int u = 0; u < NV; ++u) {
         A vx[VEC], vd[VEC];
+        if constexpr (NB < NV || NBW < NV) {
+          // (rows requested later are zeroed when their turn comes)
+          if (u >= (XW > 0 ? NBW : NB) && rows != NV && u >= rows) bd[u] = typename LV::raw_t{};
+        }
         pin(bx[u % NX]);  // one row at a time: cheap activations otherwise tempt the scheduler into unpacking many
         pin(bd[u]);       // rows ahead, which costs more registers than the tile itself
         LV::unpack(bx[u % NX], vx);
@@ -1172,6 +1194,14 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
           vd[j] = g;
         }
         bd[u] = LV::pack(vd);
+        if constexpr (XW == 0 && NB < NV) {
+          if (u + NB < NV) {
+            issue_order_fence();  // in program order behind the row just consumed
+            const int64_t o = row_offset(u + NB);
+            bx[u + NB] = LV::load(x + o);
+            bd[u + NB] = load_dy<T, VEC, DY16>(dy, o);
+          }
+        }
         if constexpr (XW > 0) {
           // the sums are brought up to date row by row: left alone, the scheduler postpones the chains of the window's
           // last rows to the end and keeps their unpacked g' alive until then
@@ -1181,9 +1211,12 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
           if constexpr (XL > 0) {
             if (u < XL) parked[u][threadIdx.x] = bx[u % NX];
           }
-          if (u + XW < NV) {
+          if (u + NBX < NV) {
             issue_order_fence();  // not before the rows ahead of it are consumed: the slot is the register budget
-            bx[u % NX] = LV::load(tile_row(x, t1, u + XW));  // the slot's next row
+            bx[(u + NBX) % NX] = LV::load(tile_row(x, t1, u + NBX));  // (its slot held row u + NBX - NX, consumed long ago)
+          }
+          if constexpr (NBW < NV) {
+            if (u + NBW < NV) bd[u + NBW] = load_dy<T, VEC, DY16>(dy_row(t1, u + NBW), 0);
           }
         }
       }
