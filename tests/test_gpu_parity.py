@@ -9,6 +9,8 @@ Tolerances (the build's stated bar):
 relu's derivative is discontinuous at 0: dx elements whose pre-activation is within RELU_BAND of 0 are
 left out of the element-wise comparison (they may legitimately land on either side).
 """
+import re
+
 import numpy as np
 import pytest
 import torch
@@ -166,6 +168,29 @@ def test_large_single_sample_backward(family, N, R, C, G, act, dtype, device):
         assert launches.get("fused_bwd") == 1 and "bwd_reduce" not in launches and "bwd_dx" not in launches, launches
     else:
         assert launches.get("bwd_dx") == 1 and "fused_bwd" not in launches, launches
+
+
+@pytest.mark.parametrize("dtype,act", [(torch.bfloat16, "silu"), (torch.float32, "gelu_tanh"), (torch.float16, "relu")])
+def test_backward_rows_requested_late_in_short_last_tiles(dtype, act, device):
+    """The single-launch backward requests four rows of a lane's tile up front and the others as rows are consumed; rows
+    past the end of a sample's last tile are masked where they are requested.  Row counts that leave the last tile's
+    lanes with 0 ... all of their rows, around the point where the late requests begin, for the tile heights the sizes
+    below select (4 to 32 rows per lane, the form that streams x through a window included), against torch in float64."""
+    seen = set()
+    before = _cabi.set_resident(True)
+    try:
+        for base in (3000, 16384, 30000, 45000, 62000):
+            for rem in (1, 33, 97, 128, 129, 161):
+                R = base - base % 32 + rem
+                print("short last tile", dtype, act, R, flush=True)
+                _check_against_torch(2, R, 320, 32, act, dtype, device)
+                inst = _cabi.last_launch()
+                m = re.search(r"fused_bwd rows=(\d+)", inst)
+                if m:
+                    seen.add(int(m.group(1)))
+    finally:
+        _cabi.set_resident(before)
+    assert len(seen) >= 3 and max(seen) >= 22, seen  # several tile heights, the tall ones among them
 
 
 def _check_against_torch(N, R, C, G, act, dtype, device):
