@@ -175,6 +175,8 @@ int gnnhwc_fwd_static(const void *x, const void *weight, const void *bias,
  * returns dx (N,R,C), dweight (C) and dbias (C).
  * Replaces run_gn_bwd_kernels<T> (gn_kernel.h:26-41; gn_kernel.cu:932-1055).
  *   dweight / dbias are written in param_dtype; either may be NULL to skip it.
+ *   dx may be the buffer of dy (every element of dy is read before the element of dx in its place is written); it must
+ *   not be the buffer of x.
  */
 int gnnhwc_bwd(const void *dy, const void *x, const void *weight, const void *bias,
                const void *mean, const void *rstd,

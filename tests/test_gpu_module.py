@@ -416,6 +416,32 @@ def test_inference_in_place_without_statistics(family, shape, G, device):
     assert torch.equal(buf, y_ref)
 
 
+@pytest.mark.parametrize("N,R,C,G,act,dtype", [
+    (2, 23 * 19, 64, 8, "silu", torch.bfloat16),
+    (4, 128 * 128, 320, 32, "gelu", torch.bfloat16),
+    (1, 150037, 192, 24, "silu", torch.bfloat16),      # the backward that keeps g' and streams x through a window
+    (6, 128 * 128, 320, 32, "relu", torch.float16),    # a backward in two launches over groups of samples
+    (3, 37 * 53, 96, 24, "gelu_tanh", torch.float32),
+    (2, 1000, 30, 5, "silu", torch.float32),           # scalar kernels
+])
+def test_backward_in_place_of_the_incoming_gradient(family, N, R, C, G, act, dtype, device):
+    """dx written into dy's own buffer (a caller that has no further use for dy) equals the ordinary call bit for bit,
+    in both kernel families."""
+    gen = torch.Generator().manual_seed(41 + R)
+    x = (torch.randn((N, R, C), generator=gen) * 1.5 + 0.3).to(dtype).to(device)
+    dy = torch.randn((N, R, C), generator=gen).to(dtype).to(device)
+    w = (torch.rand(C, generator=gen) + 0.5).to(dtype).to(device)
+    b = (0.1 * torch.randn(C, generator=gen)).to(dtype).to(device)
+    code = orc.ACT_CODES[act]
+    y, mean, rstd = cabi_fwd(x, w, b, G, 1e-5, code)
+    dx0, dw0, db0 = cabi_bwd(dy, x, w, b, mean, rstd, G, code)
+    buf = dy.clone()
+    dx1, dw1, db1 = cabi_bwd(buf, x, w, b, mean, rstd, G, code, dx=buf)
+    torch.cuda.synchronize()
+    assert dx1.data_ptr() == buf.data_ptr()
+    assert torch.equal(dx1, dx0) and torch.equal(dw1, dw0) and torch.equal(db1, db0)
+
+
 # Shapes for the recovery path of the single-launch kernels: every exchange form (all workgroups poll all tiles; two-level;
 # groups straddling chunks; partial last tiles), the backward that keeps g' only, and a backward cut into several launches
 # (its dgamma / dbeta stage reads the channel records of earlier launches).
