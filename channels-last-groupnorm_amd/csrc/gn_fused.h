@@ -633,6 +633,36 @@ __device__ __forceinline__ void recover_bwd_dx(const T *x, const T *dy, T *dx, i
   }
 }
 
+// Which channels a workgroup of the launch's first sample finishes dgamma / dbeta for.  The C channels are cut into
+// blocks of cpp channels (cpp lanes segments of a workgroup work side by side, each with as many lanes as there are
+// (sample, tile) pairs, 64 at most); block s lies in chunk s / bpc.  Workgroup (tile, chunk) takes the blocks
+// chunk * tiles + tile, that + tiles * nchunk, ...: the blocks go to the workgroups with the LOWEST linear index, the
+// first to be dispatched and the first to be done with their own rows, whatever chunk the block belongs to -- a
+// workgroup dispatched last (on a CU that serves two others first) then has nothing left to do after its dx.
+struct TailBlocks {
+  int first, stride, total;  // this workgroup's blocks: first, first + stride, ... below total
+  int bpc_log2;              // log2 of the blocks per chunk
+  int chunk_channels;        // channels of a full chunk
+};
+__device__ __forceinline__ TailBlocks tail_blocks(const Plan &p, const LanePos &l, int cpp) {
+  TailBlocks t;
+  t.chunk_channels = p.lpr * p.vec;  // a power of two (the host admits no other chunk width), as is cpp
+  const int bpc = t.chunk_channels > cpp ? t.chunk_channels >> __builtin_ctz(cpp) : 1;
+  t.bpc_log2 = __builtin_ctz(bpc);
+  t.first = l.chunk * p.tiles + l.tile;
+  t.stride = p.tiles * p.nchunk;
+  t.total = p.nchunk << t.bpc_log2;
+  return t;
+}
+// Block s: its first channel and how many of its cpp channels exist (the last chunk of a row may be narrower).
+__device__ __forceinline__ void tail_block_channels(const Plan &p, const TailBlocks &t, int s, int cpp, int &c0, int &count) {
+  const int k = s >> t.bpc_log2;
+  c0 = k * t.chunk_channels + (s & ((1 << t.bpc_log2) - 1)) * cpp;
+  const int chunk_end = (k + 1) * t.chunk_channels < (int)p.C ? (k + 1) * t.chunk_channels : (int)p.C;
+  count = chunk_end - c0 < cpp ? chunk_end - c0 : cpp;
+  if (count < 0) count = 0;
+}
+
 // dgamma / dbeta of the channels this workgroup finishes, after an expired wait of that stage: every channel record
 // of the whole tensor that feeds them is taken as it arrived, or rebuilt from x and dy.  Records of samples before n0
 // were written by launches that have ended.  x / dy point at sample n0.
@@ -646,11 +676,14 @@ __device__ __forceinline__ void recover_bwd_tail(const T *x, const T *dy, int dy
   const RecordArray rbc = channel_record_buffer(sync);
   if (threadIdx.x == 0) *sync.status = sync.epoch;
   const int pairs = (int)n_all * p.tiles;
+  const TailBlocks tb = tail_blocks(p, l, cpp);
 #pragma nounroll
-  for (int cb = l.tile * cpp; cb < l.wch; cb += p.tiles * cpp) {
+  for (int s = tb.first; s < tb.total; s += tb.stride) {
+    int c0, count;
+    tail_block_channels(p, tb, s, cpp, c0, count);
 #pragma nounroll
-    for (int cc = cb; cc < cb + cpp && cc < l.wch; ++cc) {
-      const int c = l.cstart + cc;
+    for (int cc = 0; cc < count; ++cc) {
+      const int c = c0 + cc;
       const int g = c / p.D;
       double t1 = 0.0, t2 = 0.0;
       auto slot_of = [&](int e) { return e * (int)p.C + c; };  // e = sample * tiles + tile
@@ -1359,8 +1392,11 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
     return;
   }
   const int tslot = threadIdx.x >> tlg, tsl = threadIdx.x & (TL - 1);
-  const bool tail_lane = tail && l.tile * cpp + tslot < l.wch;
-  const int tail_c = l.cstart + (tail_lane ? l.tile * cpp + tslot : 0);
+  const TailBlocks tb = tail_blocks(p, l, cpp);
+  int tail_c0 = 0, tail_count = 0;
+  if (tail && tb.first < tb.total) tail_block_channels(p, tb, tb.first, cpp, tail_c0, tail_count);
+  const bool tail_lane = tslot < tail_count;
+  const int tail_c = tail_lane ? tail_c0 + tslot : 0;
   const int tail_g = div_by(tail_c, p.by_D);
   u32x4 trec[kTailFast];
   A tmu[kTailFast], trs[kTailFast];
@@ -1424,11 +1460,12 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(fused_bw
   if (tail) {
     int spins = 0;
     late = false;
-    for (int cb = l.tile * cpp; cb < l.wch; cb += p.tiles * cpp) {
-      const bool first = cb == l.tile * cpp;
-      const int cc = cb + tslot;
-      const bool valid = cc < l.wch;
-      const int c = l.cstart + (valid ? cc : 0);
+    for (int s = tb.first; s < tb.total; s += tb.stride) {
+      const bool first = s == tb.first;
+      int c0, count;
+      tail_block_channels(p, tb, s, cpp, c0, count);
+      const bool valid = tslot < count;
+      const int c = valid ? c0 + tslot : 0;
       const int g = div_by(c, p.by_D);
       A t1 = (A)0, t2 = (A)0;
       // one (sample, tile) pair: wait until its record is this launch's (if it is this launch's to write) and add it
