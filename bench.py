@@ -293,6 +293,20 @@ def copy_ceiling(nbytes, device, steps):
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "results_all_configs.txt")
 
 
+def kernel_sources_sha16():
+    """First 16 hex digits of the SHA-256 over the kernel sources (csrc/*.h, *.hip, Makefile, in name order): what the
+    counter summary was taken on, to be compared with what is in the tree now."""
+    import glob
+    import hashlib
+
+    h = hashlib.sha256()
+    csrc = os.path.join(os.path.dirname(os.path.abspath(__file__)), "channels-last-groupnorm_amd", "csrc")
+    for path in sorted(glob.glob(os.path.join(csrc, "*.h")) + glob.glob(os.path.join(csrc, "*.hip")) + [os.path.join(csrc, "Makefile")]):
+        with open(path, "rb") as fh:
+            h.update(os.path.basename(path).encode() + b"\0" + fh.read())
+    return h.hexdigest()[:16]
+
+
 def recorded_traffic():
     """{(shape, kind): (fetch_bytes, write_bytes, instance)} from the lines `TRAFFIC <shape> <kind> <fetch> <write>
     <instance>` of the committed counter summary, or {} when there is none.  `instance` names the kernel the counters
@@ -305,6 +319,8 @@ def recorded_traffic():
                 w = ln.split()
                 if len(w) >= 5 and w[0] == "TRAFFIC":
                     out[(w[1], w[2])] = (float(w[3]), float(w[4]), w[5] if len(w) > 5 else "")
+                elif len(w) == 2 and w[0] == "SOURCES":
+                    out[("", "sources")] = w[1]  # kernel_sources_sha16() of the tree the counters were taken on
     except OSError:
         pass
     return out
@@ -1161,7 +1177,9 @@ def results_table(args, device):
         del prob
         torch.cuda.empty_cache()
     print()
-    print("machine-readable traffic per launch for bench.py (roofline.traffic), single-launch kernels only:")
+    print("machine-readable traffic per launch for bench.py (roofline.traffic), single-launch kernels only")
+    print("(SOURCES: SHA-256, first 16 digits, of the kernel sources these counters were taken on):")
+    print("SOURCES %s" % kernel_sources_sha16())
     for n in names:
         c = inst[n]
         if c["fwd_dispatches"] == 1 and c["fwd_instance"].startswith("fused"):
@@ -1271,6 +1289,8 @@ def main():
         "traffic_source": ("profiles/results_all_configs.txt (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, copy-calibrated; taken on "
                            "the kernel instance this run launches: %s)" % by_name[dom_shape].instance("bwd" if "bwd" in dominant else "fwd")
                            if tr else tr_why),
+        "traffic_taken_on_sources": traffic.get(("", "sources")),
+        "kernel_sources": kernel_sources_sha16(),
         "bytes_per_launch": dom_bytes,
         "mean_launch_us": round(dom_us, 3),
         "share_of_step": round(step_us[(dom_shape, dominant)] / total_us, 4),
